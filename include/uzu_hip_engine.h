@@ -28,7 +28,9 @@ enum {
     UZU_MODEL_DEFAULT = 0,
     UZU_MODEL_NO_GRAPH = 1,   /* decode with plain stream launches instead of hipGraph replay */
     UZU_MODEL_NO_FUSION = 2,  /* one kernel per reference kernel (no fused prologues / epilogues) */
-    UZU_MODEL_DEBUG_TAPS = 4  /* keep every layer's output of the last forward pass for inspection */
+    UZU_MODEL_DEBUG_TAPS = 4, /* keep every layer's output of the last forward pass for inspection */
+    UZU_MODEL_FULL_F32 = 8    /* an f32-stream design (uzu_model_desc::f32_stream) only: every matrix product is a true f32 product and the latent cache is f32;
+                                 default: bf16 products with f32 accumulation, bf16 cache.  UZU_ERR_UNSUPPORTED for the bf16-stream families */
 };
 /* bits 8..15 of `flags`: sequences one batched prefill pass may carry (scratch is sized for it); 0 = 1 */
 #define UZU_MODEL_BATCH(n) (((uint32_t)(n) & 0xFFu) << 8)
@@ -98,6 +100,21 @@ uzu_status uzu_hip_model_bind_state(uzu_hip_model* m, uzu_hip_state* st);
  * receives the token sampled from sequence i's last row.  The binding in force before the call is restored. */
 uzu_status uzu_hip_model_prefill_batch(uzu_hip_model* m, uzu_hip_state** states, uint32_t nseq, const uint32_t* token_ids, uint32_t count,
                                        uint32_t* first_tokens);
+/* One batched step of an f32-stream design (uzu_model_desc::f32_stream; UZU_ERR_UNSUPPORTED otherwise): sequence i appends counts[i] >= 1 tokens to states[i]
+ * (token_ids: the sequences' tokens one after the other).  Sequences of unequal length share the passes -- linears, norms and experts see one matrix of all
+ * rows, the token shift / latent cache / attention address each row's own sequence -- a prompt longer than one pass continues in the next, and more sequences
+ * than UZU_MODEL_BATCH are taken in groups.  Prefill (counts > 1, fresh or continued states) and batched decode (counts == 1) are the same call.
+ * want_rows: ascending indices into token_ids of the rows whose logits are wanted, logits_out f32 [nwant][vocab] (both may be NULL / 0).
+ * sampled_out (optional) [nseq]: the token sampled from each sequence's last row (greedy; with uzu_hip_model_set_sampling the seed of the row's position) --
+ * it also becomes that sequence's next input token, so uzu_hip_model_decode on the bound state continues from it.  A row's logits do not depend on what else
+ * the step carries or on how its prompt was cut into steps, beyond the order of f32 sums. */
+uzu_status uzu_hip_model_step_batch(uzu_hip_model* m, uzu_hip_state** states, uint32_t nseq, const uint32_t* token_ids, const uint32_t* counts,
+                                    const uint32_t* want_rows, uint32_t nwant, float* logits_out, uint32_t* sampled_out);
+/* f32 logits [vocab] of row `row` of the last pass's read-out (f32-stream designs: the last sampled row is the last one), and how many rows it produced */
+uzu_status uzu_hip_model_read_logits_f32(uzu_hip_model* m, uint32_t row, float* logits_out);
+uint32_t uzu_hip_model_logit_rows(const uzu_hip_model* m);
+/* UZU_MODEL_DEBUG_TAPS on an f32-stream design: f32 [rows, model_dim], what `layer` handed on in the last pass (`out` NULL: rows only) */
+uzu_status uzu_hip_model_read_layer_output_f32(uzu_hip_model* m, uint32_t layer, float* out, uint32_t* rows);
 /* LanguageModelState reset: context length 0, DeltaNet conv / SSM state zeroed. */
 uzu_status uzu_hip_model_reset(uzu_hip_model* m);
 uint32_t uzu_hip_model_context_length(const uzu_hip_model* m);

@@ -34,7 +34,8 @@ typedef enum {
     UZU_ACT_GELU_APPROX = 1,
     UZU_ACT_GELU_EXACT = 2,
     UZU_ACT_IDENTITY = 3,
-    UZU_ACT_SOFTPLUS = 4
+    UZU_ACT_SOFTPLUS = 4,
+    UZU_ACT_RELU_SQUARED = 5 /* max(z, 0)^2: the plain (ungated) dense MLP of an f32-stream design (uzu_layer_desc::mlp_plain) */
 } uzu_activation_type;
 
 /*
@@ -77,18 +78,33 @@ typedef struct {
 } uzu_linear_desc;
 
 /* config/normalization.rs:10-18 + tensor `scales` f32 [dim] (encodable_block/normalization.rs:67-74) */
+typedef enum {
+    UZU_NORM_STATISTICS = 0,   /* RMS / mean-variance normalisation (the reference's Normalization) */
+    UZU_NORM_DYNAMIC_TANH = 1  /* no statistics: y = tanh(alpha * x) * scales + biases, element by element (f32-stream designs) */
+} uzu_norm_kind;
 typedef struct {
     uint32_t present;       /* 0 => this optional norm is absent */
     uint32_t full_layer;    /* UpcastMode::FullLayer (1) vs OnlyNormalization (0) */
     uint32_t subtract_mean; /* LayerNorm-style mean subtraction */
-    uint32_t reserved;
+    uint32_t kind;          /* uzu_norm_kind (the field was `reserved`: 0 = the reference's Normalization) */
     float epsilon;
     float scale_offset;     /* Option<f32>::unwrap_or(0.0) */
     const float* scales;    /* f32 [dim] or NULL (has_scale == false) */
     const float* biases;    /* f32 [dim] or NULL */
+    float alpha;            /* UZU_NORM_DYNAMIC_TANH: the scalar inside the tanh */
+    uint32_t reserved;
 } uzu_norm_desc;
 
-typedef enum { UZU_MIXER_ATTENTION = 0, UZU_MIXER_DELTA_NET = 1 } uzu_mixer_kind;
+typedef enum {
+    UZU_MIXER_ATTENTION = 0,
+    UZU_MIXER_DELTA_NET = 1,
+    /* Attention over a cached low-rank latent (f32-stream designs): per token only c = RMSNorm(W_down h) [latent_rank] is kept; a head's keys and values are
+     * W_up_k c and W_up_v c, so scores and the weighted sum run in latent space (q W_up_k applied to the query, W_up_v to the result).  No rotation.  Reuses the
+     * attention fields: num_heads, head_dim (query / key width per head), attention_scale, sliding_window_size, has_sinks / sinks, is_kv_sharing +
+     * kv_source_layer_index (the sharing layer reads the source layer's cached latents through its OWN up projections), qkv_projection (queries only,
+     * n = heads * head_dim), out_projection (k = heads * value_head_dim); and the latent_* fields at the end of uzu_layer_desc. */
+    UZU_MIXER_LATENT_ATTENTION = 2
+} uzu_mixer_kind;
 
 /* config/rope/*.rs -- every AnyRoPEConfig variant (encodable_block/mixer/attention/rope.rs:13-114) */
 typedef enum { UZU_ROPE_NONE = 0, UZU_ROPE_UNSCALED = 1, UZU_ROPE_LLAMA = 2, UZU_ROPE_LINEAR = 3, UZU_ROPE_YARN = 4,
@@ -131,7 +147,15 @@ typedef struct {
     const uint16_t* w2;
     const uint16_t* up_biases;
     const uint16_t* down_biases;
+    /* Score routing (f32-stream designs; routing == UZU_MOE_ROUTE_SCORES): scores = softmax of the router logits over ALL num_routed_experts +
+     * num_identity_experts outputs; the num_active_experts largest (score + selection_bias) win; a winner's weight is its score divided by the winners'
+     * score sum (+ 1e-20).  The last num_identity_experts router outputs have no tensors: such an expert returns its input.  No router / expert biases
+     * (the bias pointers are NULL); router_weights is [routed + identity, model_dim]. */
+    uint32_t routing;              /* uzu_moe_routing; 0 = the reference's top-k of the logits */
+    uint32_t num_identity_experts;
+    const float* selection_bias;   /* f32 [routed + identity]: added to the scores for the choice only */
 } uzu_moe_desc;
+typedef enum { UZU_MOE_ROUTE_TOPK_LOGITS = 0, UZU_MOE_ROUTE_SCORES = 1 } uzu_moe_routing;
 
 typedef enum { UZU_MLP_DENSE = 0, UZU_MLP_MOE = 1 } uzu_mlp_kind;
 
@@ -206,6 +230,23 @@ typedef struct {
 
     /* --- mixture of experts (mlp_kind == UZU_MLP_MOE: up_projection / down_projection / hidden_dim / activation above are unused) --- */
     uzu_moe_desc moe;
+
+    /* --- layer mechanisms of the f32-stream designs (uzu_model_desc::f32_stream); all zero / NULL = none --- */
+    uint32_t latent_rank;        /* UZU_MIXER_LATENT_ATTENTION: width of the cached latent */
+    uint32_t value_head_dim;     /* ... value width per head (out_projection.k = num_heads * value_head_dim) */
+    uzu_linear_desc latent_down;      /* n = latent_rank, k = model_dim; absent (weights NULL) on a sharing layer */
+    uzu_norm_desc latent_norm;        /* RMS norm of the latent, scales [latent_rank]; absent on a sharing layer */
+    uzu_linear_desc latent_up_keys;   /* n = num_heads * head_dim, k = latent_rank */
+    uzu_linear_desc latent_up_values; /* n = num_heads * value_head_dim, k = latent_rank */
+    /* Token shift: the mixer reads h + (h_prev - h) * token_shift, h_prev = the previous position's normalised row before this replacement (zeros at
+     * position 0); the last row's h is part of the sequence state. */
+    const float* token_shift;    /* f32 [model_dim] or NULL */
+    /* Depth mix: with X_0 the embedding rows and X_(j+1) layer j's own result, what layer l hands on is sum_{j <= l+1} depth_weights[j] * X_j. */
+    const float* depth_weights;  /* f32 [num_depth_weights] or NULL */
+    uint32_t num_depth_weights;  /* l + 2 on layer l */
+    uint32_t mlp_plain;          /* dense MLP without a gate: down(act(up x + b) ) + b, up_projection.n == hidden_dim */
+    uint32_t no_mlp;             /* the layer ends behind its mixer */
+    uint32_t reserved4;
 } uzu_layer_desc;
 
 typedef struct {
@@ -242,6 +283,12 @@ typedef struct {
     uzu_linear_desc ple_model_projection; /* per_layer_embedding.model_projection: n = num_layers*ple_dim, k = model_dim */
     uzu_norm_desc ple_projection_norm;    /* per_layer_embedding.projection_norm: [ple_dim]; epsilon as configured (the engine divides it by
                                              model_projection_scale^2, per_layer_embedding.rs:75-80) */
+    /* An f32-stream design: the residual stream, norms, attention scores / weights and routers are f32 end to end (the reference's models re-round the residual
+     * to bf16 at every add); weights are full-precision bf16 (UZU_QUANT_NONE); pre-norm layers x <- x + mixer(norm(x)), x <- x + mlp(norm(x)); the read-out is the
+     * tied embedding table behind output_norm; logits are f32.  Such a model runs through its own forward encoder (csrc/engine_stream32.hip), batched over
+     * sequences of unequal length (uzu_hip_model_step_batch). */
+    uint32_t f32_stream;
+    uint32_t reserved5;
 } uzu_model_desc;
 
 /*

@@ -14,6 +14,7 @@
 // the next input token and the sampled-token history live in device memory, so ONE captured hipGraph is
 // replayed for every decode step and steps are chained without a host round trip.
 #include "engine_types.h"
+#include "uzu_math.h"
 
 using namespace uzu;
 using namespace uzu::eng;
@@ -32,6 +33,12 @@ static void drop_pending_tree(uzu_hip_model* m, const uzu_hip_state* moving) {
 uzu_status uzu_hip_model_prefill_batch(uzu_hip_model* m, uzu_hip_state** states, uint32_t nseq, const uint32_t* token_ids, uint32_t count,
                                        uint32_t* first_tokens) {
     UZU_REQUIRE(m && states && token_ids && nseq > 0 && count > 0, "model_prefill_batch: null / empty input");
+    if (m->s32) { // an f32-stream design: the batched step with equal counts
+        std::vector<uint32_t> counts(nseq, count), sampled(nseq);
+        UZU_PROPAGATE(s32_step_batch(m, states, nseq, token_ids, counts.data(), nullptr, 0, nullptr, sampled.data()));
+        if (first_tokens) memcpy(first_tokens, sampled.data(), (size_t)nseq * 4);
+        return UZU_OK;
+    }
     UZU_REQUIRE(nseq <= m->max_seqs, "model_prefill_batch: %u sequences, model created for at most %u (UZU_MODEL_BATCH)", nseq, m->max_seqs);
     for (uint32_t i = 0; i < nseq; ++i) {
         UZU_REQUIRE(states[i] && states[i]->m == m, "model_prefill_batch: state %u is null or belongs to another model", i);
@@ -110,6 +117,7 @@ uzu_status uzu_hip_model_prefill(uzu_hip_model* m, const uint32_t* token_ids, ui
     UZU_REQUIRE(m && token_ids && count > 0, "model_prefill: null / empty input");
     UZU_REQUIRE(m->context_length + count <= m->d.max_context_length, "model_prefill: %u + %u tokens exceed max_context_length %u",
                 m->context_length, count, m->d.max_context_length);
+    if (m->s32) return s32_prefill(m, token_ids, count, first_token);
     hipStream_t s = m->ctx->stream;
     m->hidden_ready = false; // the prefill pass uses `hidden` for its own rows
     drop_pending_tree(m, m->bound);
@@ -144,6 +152,7 @@ static void drop_stale_graphs(uzu_hip_model* m);
 uzu_status uzu_hip_model_decode_enqueue(uzu_hip_model* m, uint32_t steps) {
     UZU_REQUIRE(m, "model_decode: null model");
     UZU_REQUIRE(m->context_length > 0, "model_decode: prefill first (no input token)");
+    if (m->s32) return s32_decode_enqueue(m, steps);
     drop_stale_graphs(m);
     drop_pending_tree(m, m->bound);
     return enqueue_decode(m, steps);
@@ -165,7 +174,7 @@ uzu_status uzu_hip_model_decode(uzu_hip_model* m, uint32_t steps, uint32_t* out_
     if (!steps) return UZU_OK;
     // make sure graph construction is not inside the timed region
     drop_stale_graphs(m);
-    if (!(m->flags & UZU_MODEL_NO_GRAPH) && !k::exact_mode()) {
+    if (!(m->flags & UZU_MODEL_NO_GRAPH) && !k::exact_mode() && !m->s32) {
         if (m->context_length + 1 <= 1024 && !m->graph_single) UZU_PROPAGATE(build_decode_graph(m, &m->graph_single, false));
         if (m->context_length + steps > 1024 && !m->graph_two) UZU_PROPAGATE(build_decode_graph(m, &m->graph_two, true));
     }
@@ -182,8 +191,27 @@ uzu_status uzu_hip_model_decode(uzu_hip_model* m, uint32_t steps, uint32_t* out_
     return UZU_OK;
 }
 
+uzu_status uzu_hip_model_step_batch(uzu_hip_model* m, uzu_hip_state** states, uint32_t nseq, const uint32_t* token_ids, const uint32_t* counts,
+                                    const uint32_t* want_rows, uint32_t nwant, float* logits_out, uint32_t* sampled_out) {
+    UZU_REQUIRE(m && states && token_ids && counts && nseq > 0, "model_step_batch: null / empty input");
+    UZU_UNSUPPORTED(!m->s32, "model_step_batch: batched steps of unequal sequences are a path of the f32-stream designs (this model: uzu_hip_model_prefill_batch + decode per state)");
+    return s32_step_batch(m, states, nseq, token_ids, counts, want_rows, nwant, logits_out, sampled_out);
+}
+uzu_status uzu_hip_model_read_logits_f32(uzu_hip_model* m, uint32_t row, float* logits_out) {
+    UZU_REQUIRE(m && logits_out, "model_read_logits_f32: null argument");
+    UZU_UNSUPPORTED(!m->s32, "model_read_logits_f32: this model's logits are bf16 (uzu_hip_model_read_logits)");
+    return s32_read_logits_f32(m, logits_out, row);
+}
+uint32_t uzu_hip_model_logit_rows(const uzu_hip_model* m) { return m && m->s32 ? s32_last_logit_rows(m) : (m ? 1u : 0u); }
+uzu_status uzu_hip_model_read_layer_output_f32(uzu_hip_model* m, uint32_t layer, float* out, uint32_t* rows) {
+    UZU_REQUIRE(m, "model_read_layer_output_f32: null model");
+    UZU_UNSUPPORTED(!m->s32, "model_read_layer_output_f32: this model's taps are bf16 (uzu_hip_model_read_layer_output)");
+    return s32_read_layer_output(m, layer, out, rows);
+}
+
 uzu_status uzu_hip_model_profile_decode_step(uzu_hip_model* m, uint32_t capacity, const char** names, uint64_t* bytes, float* ms, uint32_t* count) {
     UZU_REQUIRE(m && names && bytes && ms && count, "model_profile_decode_step: null argument");
+    UZU_UNSUPPORTED(m->s32 != nullptr, "model_profile_decode_step: the per-launch profile reads the bf16-stream decode step");
     UZU_REQUIRE(m->context_length > 0 && m->context_length + 1 <= m->d.max_context_length, "model_profile_decode_step: bad context length");
     std::vector<ProfEntry> prof;
     m->prof_sink = &prof;
@@ -253,6 +281,13 @@ uzu_status uzu_hip_model_set_next_token(uzu_hip_model* m, uint32_t token) {
 
 uzu_status uzu_hip_model_read_logits(uzu_hip_model* m, uint16_t* logits_out) {
     UZU_REQUIRE(m && logits_out, "model_read_logits: null argument");
+    if (m->s32) { // f32 logits: the last row of the last read-out, rounded for this entry point
+        std::vector<float> row(m->d.vocab_size);
+        UZU_REQUIRE(s32_last_logit_rows(m) > 0, "model_read_logits: no logits yet");
+        UZU_PROPAGATE(s32_read_logits_f32(m, row.data(), s32_last_logit_rows(m) - 1));
+        for (uint32_t i = 0; i < m->d.vocab_size; ++i) logits_out[i] = f32_to_bf16(row[i]);
+        return UZU_OK;
+    }
     HIPCHK(hipStreamSynchronize(m->ctx->stream));
     HIPCHK(hipMemcpy(logits_out, m->logits, (size_t)(m->d.tied_embeddings ? m->embedding.n : m->output_embedding.n) * 2, hipMemcpyDeviceToHost));
     return UZU_OK;
@@ -320,6 +355,7 @@ uzu_status uzu_hip_model_verify_tree(uzu_hip_model* m, const uint32_t* token_ids
 uzu_status uzu_hip_model_verify_tree_seeded(uzu_hip_model* m, const uint32_t* token_ids, const uint32_t* trie_nodes, const uint64_t* seeds, uint32_t tree_size,
                                             uint32_t* sampled_out) {
     UZU_REQUIRE(m && token_ids && trie_nodes && tree_size > 0, "model_verify_tree: null / empty input");
+    UZU_UNSUPPORTED(m->s32 != nullptr, "model_verify_tree: speculative tree passes are not built for the f32-stream designs");
     (void)hipSetDevice(m->ctx->device);
     UZU_UNSUPPORTED(tree_size > k::kDnTreeMaxNodes, "model_verify_tree: %u nodes (at most %u per pass)", tree_size, k::kDnTreeMaxNodes);
     UZU_REQUIRE(m->tree.size == 0, "model_verify_tree: a speculated tree is already pending (accept it first)");

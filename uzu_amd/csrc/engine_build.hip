@@ -106,7 +106,9 @@ uzu_status state_build(uzu_hip_model* m, uzu_hip_state** out) {
     for (size_t l = 0; l < m->layers.size(); ++l) {
         const uzu_layer_desc& h = m->layers[l].d;
         void* p = nullptr;
-        if (h.mixer_kind == UZU_MIXER_ATTENTION && h.is_kv_sharing) {
+        if (h.mixer_kind == UZU_MIXER_LATENT_ATTENTION) {
+            if (r == UZU_OK) r = s32_state_layer(m, st, (uint32_t)l); // latent cache (unless shared) + the token shift's row
+        } else if (h.mixer_kind == UZU_MIXER_ATTENTION && h.is_kv_sharing) {
             // TransformerLayerStateType::Shared(kv_source_layer_index) (transformer.rs:205-216): no state of its own
         } else if (h.mixer_kind == UZU_MIXER_ATTENTION) {
             // AttentionState::create_empty (state.rs:69-136): a causal sliding-window layer keeps a RING of `window` rows + the suffix region
@@ -318,6 +320,16 @@ uzu_status uzu_hip_model_create_tp(uzu_hip_context* ctx, const uzu_model_desc* d
                                    uzu_hip_model** out) {
     UZU_REQUIRE(ctx && desc && out, "model_create: null argument");
     UZU_REQUIRE(desc->num_layers > 0 && desc->layers, "model_create: no layers");
+    if (desc->f32_stream) { // its own builder and forward encoder (engine_stream32.hip); the model / state objects and the C ABI are the same
+        UZU_UNSUPPORTED(comm != nullptr, "model_create: f32-stream designs are not sharded (single GPU only)");
+        return s32_create(ctx, desc, flags, out);
+    }
+    UZU_UNSUPPORTED(flags & UZU_MODEL_FULL_F32, "model_create: UZU_MODEL_FULL_F32 is a precision of the f32-stream designs; this model's stream is bf16");
+    for (uint32_t l = 0; l < desc->num_layers; ++l)
+        UZU_UNSUPPORTED(desc->layers[l].mixer_kind == UZU_MIXER_LATENT_ATTENTION || desc->layers[l].token_shift || desc->layers[l].depth_weights || desc->layers[l].mlp_plain ||
+                        desc->layers[l].no_mlp || desc->layers[l].pre_mixer_norm.kind != UZU_NORM_STATISTICS || desc->layers[l].pre_mlp_norm.kind != UZU_NORM_STATISTICS ||
+                        (desc->layers[l].mlp_kind == UZU_MLP_MOE && desc->layers[l].moe.routing != UZU_MOE_ROUTE_TOPK_LOGITS),
+                        "model_create: layer %u uses a mechanism of the f32-stream designs (set uzu_model_desc::f32_stream)", l);
     (void)hipSetDevice(ctx->device);
     auto* m = new uzu_hip_model();
     m->ctx = ctx;
@@ -689,6 +701,7 @@ void uzu_hip_model_destroy(uzu_hip_model* m) {
     if (m->ev1) (void)hipEventDestroy(m->ev1);
     for (void* p : m->allocations) (void)hipFree(p);
     for (size_t b : m->allocation_bytes) m->ctx->current_bytes -= b < m->ctx->current_bytes ? b : m->ctx->current_bytes;
+    if (m->s32) s32_destroy(m);
     delete m;
 }
 

@@ -68,6 +68,7 @@ extern "C" {
 // ---- the target's hidden-feature taps ----------------------------------------------------------------------------------------------------------------
 uzu_status uzu_hip_model_set_feature_layers(uzu_hip_model* m, const uint32_t* layer_ids, uint32_t count) {
     UZU_REQUIRE(m && (layer_ids || !count), "model_set_feature_layers: null argument");
+    UZU_UNSUPPORTED(m->s32 != nullptr && count, "model_set_feature_layers: hidden-feature taps of an f32-stream design");
     UZU_UNSUPPORTED(m->tp != nullptr && count, "model_set_feature_layers: hidden-feature taps of a tensor-parallel shard");
     for (uint32_t i = 0; i < count; ++i) UZU_REQUIRE(layer_ids[i] < m->d.num_layers, "model_set_feature_layers: layer %u of %u", layer_ids[i], m->d.num_layers);
     (void)hipSetDevice(m->ctx->device);
@@ -116,6 +117,7 @@ void uzu_hip_drafter_destroy(uzu_hip_drafter* f) {
 
 uzu_status uzu_hip_drafter_create(uzu_hip_context* ctx, uzu_hip_model* target, const uzu_dflash_desc* desc, uzu_hip_drafter** out) {
     UZU_REQUIRE(ctx && target && desc && out, "drafter_create: null argument");
+    UZU_UNSUPPORTED(target->s32 != nullptr, "drafter_create: a draft model on an f32-stream target");
     UZU_REQUIRE(desc->num_layers > 0 && desc->layers && desc->num_target_layers > 0 && desc->target_layer_ids, "drafter_create: no layers / no target layers");
     UZU_REQUIRE(desc->model_dim == target->d.model_dim, "drafter_create: draft model_dim %u != target model_dim %u (the draft model embeds through the target's table)", desc->model_dim,
                 target->d.model_dim);

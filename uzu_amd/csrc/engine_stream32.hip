@@ -1,0 +1,570 @@
+// engine_stream32.hip -- the forward encoder of the f32-stream designs (uzu_model_desc::f32_stream; first family: Lazolix).
+//
+// What differs from the reference's models (engine_forward.hip): the residual stream stays f32 from the embedding to the read-out (nothing is re-rounded to
+// bf16 between layers), norms are dynamic-tanh norms, a layer's mixer reads token-shifted rows, the mixer is attention over a cached low-rank latent
+// (k_latent_attention.hip), the MLP is a plain dense block or score-routed experts with identity experts, every layer ends in a depth mix over the results of
+// all layers before it, and logits are f32.  What is shared: the model / state objects and their memory accounting (engine_build.hip), the sampling kernels,
+// the device-resident control block (context length, next token, sampled history) and the C ABI above (engine_api.hip).
+//
+// A pass carries rows of SEVERAL sequences of unequal length (struct k::SeqSpan): linears, norms and experts see one matrix of all rows; the token shift, the
+// latent cache and the attention core address each row's own sequence through pointer tables built per pass.  A prompt longer than one pass (m->chunk rows)
+// continues in the next pass from the state the previous one left: the cache rows and the last normalised row per layer.
+//
+// Precisions: `bf16_products` (default) rounds the activation operand of every matrix product to bf16 and keeps the latent cache in bf16; UZU_MODEL_FULL_F32
+// makes every product a true f32 product and the cache f32.  Everything else is f32 either way.
+#include <algorithm>
+
+#include "engine_types.h"
+#include "kernels_stream32.h"
+#include "uzu_math.h"
+
+using namespace uzu;
+using namespace uzu::eng;
+
+namespace uzu {
+namespace eng {
+
+struct Stream32 {
+    bool full_f32 = false;
+    uint32_t max_rows = 0, max_seqs = 1;
+    float *slots = nullptr, *xin = nullptr, *normed = nullptr, *q = nullptr, *ckv = nullptr, *qlat = nullptr, *ctx = nullptr, *attn = nullptr, *hid = nullptr;
+    int32_t* moe_ids = nullptr;
+    float* moe_w = nullptr;
+    float *out_normed = nullptr, *logits = nullptr;
+    size_t logit_rows = 0;
+    k::SeqSpan* d_spans = nullptr;
+    uint32_t *d_row_seq = nullptr, *d_out_rows = nullptr;
+    void** d_cache_ptrs = nullptr;  // [layers][max_seqs]
+    float** d_shift_ptrs = nullptr; // [layers][max_seqs]
+    struct Layer {
+        uint16_t* up_keys_t = nullptr; // bf16 [heads][rank][head_dim]: W_up_k of a head transposed, so that folding it into the query is an ordinary product
+        float* sinks = nullptr;        // f32 [heads]
+        float *token_shift = nullptr, *depth_weights = nullptr, *selection_bias = nullptr;
+        float alpha1 = 0.f, alpha2 = 0.f;
+    };
+    std::vector<Layer> layers;
+    float alpha_out = 0.f;
+    float* taps = nullptr; // UZU_MODEL_DEBUG_TAPS: f32 [layers][max_rows][d], what each layer handed on in the last pass
+    uint32_t tap_rows = 0;
+    uint32_t last_logit_rows = 0; // rows of `logits` the last pass produced
+};
+
+namespace {
+
+uint32_t state_length(const uzu_hip_model* m, const uzu_hip_state* st) { return m->bound == st ? m->context_length : st->context_length; }
+void state_set_length(uzu_hip_model* m, uzu_hip_state* st, uint32_t len) {
+    st->context_length = len;
+    if (m->bound == st) m->context_length = len;
+}
+
+__global__ void s32_commit_kernel(uint32_t* ctx_len, uint32_t* tokens, const uint32_t* out_token, uint32_t* sampled, uint32_t count, uint32_t has_token) {
+    const uint32_t len = *ctx_len;
+    if (has_token) {
+        const uint32_t t = *out_token;
+        sampled[len + count - 1] = t;
+        tokens[0] = t;
+    }
+    *ctx_len = len + count;
+}
+
+uzu_status need_f32(uzu_hip_model* m, size_t floats, float** out) {
+    void* p = nullptr;
+    UZU_PROPAGATE(dev_alloc(m, floats * 4, &p, true));
+    *out = (float*)p;
+    return UZU_OK;
+}
+
+struct PassSeq {
+    uzu_hip_state* st;
+    uint32_t count, start;
+};
+
+k::LinearF32Params lin(const Stream32& S, const DLinear& L, const float* x, float* y, uint32_t rows) {
+    k::LinearF32Params p{};
+    p.x = x, p.w = (const uint16_t*)L.w, p.bias = (const uint16_t*)L.out_biases, p.y = y;
+    p.rows = rows, p.n = L.n, p.k = L.k, p.ldx = L.k, p.ldy = L.n, p.ldr = L.n, p.batch = 1;
+    p.bf16_products = S.full_f32 ? 0u : 1u;
+    return p;
+}
+
+void run_linear(Enc& e, const k::LinearF32Params& p) {
+    const char* variant = "linear_f32";
+    e.begin();
+    const uzu_status r = k::linear_f32(e.s, p, &variant);
+    e.run(r, variant, k::linear_f32_bytes(p));
+}
+
+// One pass over `seqs` (rows = sum of their counts, <= max_rows; token ids on the device, row-major in sequence order).  `out_rows`: rows of the pass whose
+// logits are wanted, in order; they land in S.logits [out_rows.size()][vocab] f32.  Does not move the sequences' context lengths.
+uzu_status s32_pass(uzu_hip_model* m, const std::vector<PassSeq>& seqs, const uint32_t* d_tokens, const std::vector<uint32_t>& out_rows) {
+    Stream32& S = *m->s32;
+    hipStream_t s = m->ctx->stream;
+    Enc e{m, s};
+    e.prof = (std::vector<ProfEntry>*)m->prof_sink;
+    m->launches = 0;
+    const uint32_t d = m->d.model_dim, nl = m->d.num_layers, nseq = (uint32_t)seqs.size();
+    UZU_REQUIRE(nseq > 0 && nseq <= S.max_seqs, "engine: a pass of %u sequences (the model carries at most %u)", nseq, S.max_seqs);
+    std::vector<k::SeqSpan> spans(nseq);
+    std::vector<uint32_t> row_seq;
+    uint32_t rows = 0;
+    for (uint32_t i = 0; i < nseq; ++i) {
+        spans[i] = {rows, seqs[i].count, seqs[i].start};
+        UZU_REQUIRE(seqs[i].count > 0 && seqs[i].start + seqs[i].count <= m->max_positions, "engine: sequence %u leaves its state's capacity", i);
+        for (uint32_t j = 0; j < seqs[i].count; ++j) row_seq.push_back(i);
+        rows += seqs[i].count;
+    }
+    UZU_REQUIRE(rows <= S.max_rows, "engine: a pass of %u rows (at most %u)", rows, S.max_rows);
+    std::vector<void*> cache_ptrs((size_t)nl * S.max_seqs, nullptr);
+    std::vector<float*> shift_ptrs((size_t)nl * S.max_seqs, nullptr);
+    for (uint32_t l = 0; l < nl; ++l) {
+        const uzu_layer_desc& h = m->layers[l].d;
+        const uint32_t src = h.is_kv_sharing ? h.kv_source_layer_index : l;
+        for (uint32_t i = 0; i < nseq; ++i) {
+            cache_ptrs[(size_t)l * S.max_seqs + i] = seqs[i].st->layers[src].latent;
+            shift_ptrs[(size_t)l * S.max_seqs + i] = seqs[i].st->layers[l].shift_prev;
+        }
+    }
+    // (pageable sources: the copies have left the host buffers when the calls return)
+    HIPCHK(hipMemcpyAsync(S.d_spans, spans.data(), spans.size() * sizeof(k::SeqSpan), hipMemcpyHostToDevice, s));
+    HIPCHK(hipMemcpyAsync(S.d_row_seq, row_seq.data(), row_seq.size() * 4, hipMemcpyHostToDevice, s));
+    HIPCHK(hipMemcpyAsync(S.d_cache_ptrs, cache_ptrs.data(), cache_ptrs.size() * sizeof(void*), hipMemcpyHostToDevice, s));
+    HIPCHK(hipMemcpyAsync(S.d_shift_ptrs, shift_ptrs.data(), shift_ptrs.size() * sizeof(float*), hipMemcpyHostToDevice, s));
+    if (!out_rows.empty()) HIPCHK(hipMemcpyAsync(S.d_out_rows, out_rows.data(), out_rows.size() * 4, hipMemcpyHostToDevice, s));
+
+    const size_t slot_stride = (size_t)S.max_rows * d;
+    const uint32_t bf = S.full_f32 ? 0u : 1u;
+    RUN("embed_rows_f32", (size_t)rows * d * 6, k::embed_rows_f32(s, d_tokens, (const uint16_t*)m->embedding.w, S.slots, rows, m->d.vocab_size, d));
+    const float* cur = S.slots; // what the layer about to run reads: X_0, then the depth mix of the layer before
+    for (uint32_t l = 0; l < nl; ++l) {
+        DLayer& L = m->layers[l];
+        const Stream32::Layer& X = S.layers[l];
+        const uzu_layer_desc& h = L.d;
+        float* slot = S.slots + (size_t)(l + 1) * slot_stride; // X_(l+1): the layer's own result
+        void* const* caches = S.d_cache_ptrs + (size_t)l * S.max_seqs;
+        {   // pre-mixer norm + token shift
+            k::DynTanhParams np{};
+            np.x = cur, np.out = S.normed, np.scales = L.pre_mixer.scales, np.biases = L.pre_mixer.biases, np.alpha = X.alpha1, np.shift = X.token_shift;
+            np.spans = S.d_spans, np.row_seq = S.d_row_seq, np.prev = S.d_shift_ptrs + (size_t)l * S.max_seqs, np.rows = rows, np.d = d;
+            RUN("dyn_tanh_norm+shift", (size_t)rows * d * 8, k::dyn_tanh_norm(s, np));
+        }
+        const uint32_t H = h.num_heads, hd = h.head_dim, vd = h.value_head_dim, rank = h.latent_rank;
+        run_linear(e, lin(S, L.qkv, S.normed, S.q, rows));
+        if (!h.is_kv_sharing) {
+            run_linear(e, lin(S, L.lat_down, S.normed, S.ckv, rows));
+            RUN("latent_norm_append", (size_t)rows * rank * 6,
+                k::latent_norm_append(s, S.ckv, L.lat_norm.scales, L.lat_norm.eps, caches, bf, S.d_spans, S.d_row_seq, rows, rank));
+        }
+        {   // the head's key projection folded into the query: qlat[r, h, :] = W_up_k[h]^T q[r, h, :]
+            k::LinearF32Params p{};
+            p.x = S.q, p.w = X.up_keys_t, p.y = S.qlat, p.rows = rows, p.n = rank, p.k = hd, p.ldx = H * hd, p.ldy = H * rank, p.batch = H;
+            p.x_batch = hd, p.w_batch = (size_t)rank * hd, p.y_batch = rank, p.bf16_products = bf;
+            run_linear(e, p);
+        }
+        {
+            k::LatentAttentionParams ap{};
+            ap.qlat = S.qlat, ap.out = S.ctx, ap.caches = caches, ap.cache_bf16 = bf, ap.sinks = X.sinks, ap.spans = S.d_spans, ap.row_seq = S.d_row_seq;
+            ap.rows = rows, ap.heads = H, ap.rank = rank, ap.window = h.sliding_window_size;
+            ap.scale = h.attention_scale != 0.0f ? h.attention_scale : 1.0f / sqrtf((float)hd);
+            RUN("latent_attention", (size_t)rows * H * rank * 8, k::latent_attention(s, ap));
+        }
+        {   // the head's value projection on the weighted latent sum: attn[r, h, :] = W_up_v[h] ctx[r, h, :]
+            k::LinearF32Params p{};
+            p.x = S.ctx, p.w = (const uint16_t*)L.lat_up_v.w, p.y = S.attn, p.rows = rows, p.n = vd, p.k = rank, p.ldx = H * rank, p.ldy = H * vd, p.batch = H;
+            p.x_batch = rank, p.w_batch = (size_t)vd * rank, p.y_batch = vd, p.bf16_products = bf;
+            run_linear(e, p);
+        }
+        {   // X_(l+1) = input + out projection
+            k::LinearF32Params p = lin(S, L.out, S.attn, slot, rows);
+            p.residual = cur, p.ldr = d;
+            run_linear(e, p);
+        }
+        if (!h.no_mlp) {
+            k::DynTanhParams np{};
+            np.x = slot, np.out = S.normed, np.scales = L.pre_mlp.scales, np.biases = L.pre_mlp.biases, np.alpha = X.alpha2, np.rows = rows, np.d = d;
+            RUN("dyn_tanh_norm", (size_t)rows * d * 8, k::dyn_tanh_norm(s, np));
+            if (h.mlp_kind == UZU_MLP_MOE) {
+                const uzu_moe_desc& M = h.moe;
+                const uint32_t E = M.num_routed_experts, top = M.num_active_experts, ff = M.expert_hidden_dim;
+                RUN("moe_route_scores", (size_t)(E + M.num_identity_experts) * d * 2,
+                    k::moe_route_scores(s, S.normed, L.moe.router_weights, X.selection_bias, S.moe_ids, S.moe_w, rows, d, E + M.num_identity_experts, top));
+                RUN("moe_experts_gate_up", (size_t)rows * top * 2 * ff * d * 2, k::moe_experts_gate_up(s, S.normed, S.moe_ids, L.moe.w13, S.hid, rows, d, ff, E, top, bf));
+                RUN("moe_experts_down_combine", (size_t)rows * top * ff * d * 2,
+                    k::moe_experts_down_combine(s, S.hid, S.normed, S.moe_ids, S.moe_w, L.moe.w2, slot, slot, rows, d, ff, E, top, bf));
+            } else {
+                k::LinearF32Params up = lin(S, L.up, S.normed, S.hid, rows);
+                up.act = 1;
+                run_linear(e, up);
+                k::LinearF32Params down = lin(S, L.down, S.hid, slot, rows);
+                down.residual = slot, down.ldr = d;
+                run_linear(e, down);
+            }
+        }
+        if (X.depth_weights) {
+            RUN("depth_mix", (size_t)rows * d * 4 * (l + 3), k::depth_mix(s, S.slots, slot_stride, X.depth_weights, h.num_depth_weights, S.xin, rows, d));
+            cur = S.xin;
+        } else {
+            cur = slot;
+        }
+        if (S.taps) HIPCHK(hipMemcpyAsync(S.taps + (size_t)l * slot_stride, cur, (size_t)rows * d * 4, hipMemcpyDeviceToDevice, s));
+    }
+    S.tap_rows = rows;
+    S.last_logit_rows = 0;
+    if (!out_rows.empty()) {
+        const uint32_t n_out = (uint32_t)out_rows.size();
+        k::DynTanhParams np{};
+        np.x = cur, np.out = S.out_normed, np.scales = m->output_norm.scales, np.biases = m->output_norm.biases, np.alpha = S.alpha_out, np.row_index = S.d_out_rows;
+        np.rows = n_out, np.d = d;
+        RUN("dyn_tanh_norm", (size_t)n_out * d * 8, k::dyn_tanh_norm(s, np));
+        run_linear(e, lin(S, m->embedding, S.out_normed, S.logits, n_out));
+        S.last_logit_rows = n_out;
+    }
+    if (e.st != UZU_OK) return e.st;
+    const hipError_t herr = hipGetLastError();
+    if (herr != hipSuccess) {
+        set_error("engine: f32-stream pass launch failed: %s", hipGetErrorString(herr));
+        return UZU_ERR_HIP;
+    }
+    return UZU_OK;
+}
+
+uzu_status ensure_logits(uzu_hip_model* m, size_t rows) {
+    Stream32& S = *m->s32;
+    if (rows <= S.logit_rows) return UZU_OK;
+    HIPCHK(hipStreamSynchronize(m->ctx->stream));
+    if (S.logits) dev_free(m, S.logits);
+    S.logits = nullptr, S.logit_rows = 0;
+    size_t want = rows < 16 ? 16 : rows;
+    void* p = nullptr;
+    UZU_PROPAGATE(dev_alloc(m, want * m->d.vocab_size * 4, &p));
+    S.logits = (float*)p, S.logit_rows = want;
+    return UZU_OK;
+}
+
+// sample from row `logit_row` of the last pass's logits into st's control block and advance it by `count`
+uzu_status sample_commit(uzu_hip_model* m, uzu_hip_state* st, uint32_t logit_row, uint32_t count, bool sample) {
+    Stream32& S = *m->s32;
+    hipStream_t s = m->ctx->stream;
+    Enc e{m, s};
+    if (sample) {
+        const float* row = S.logits + (size_t)logit_row * m->d.vocab_size;
+        if (m->sampling.on) { // the seed of the sampled row's position, as in the engine's other models
+            RUN("derive_seed", 0, k::derive_seed(s, m->sampling.seed, st->d_ctx_len, count - 1, m->d_seed));
+            k::UnifiedSamplingParams sp = m->sampling.p;
+            sp.logits = row, sp.dt = UZU_F32, sp.output = st->d_out_token, sp.seeds = m->d_seed, sp.vocab_size = m->d.vocab_size, sp.batch_size = 1;
+            RUN("unified_sampling", (size_t)sp.vocab_size * 4, k::unified_sampling(s, sp, m->sampling_scratch));
+        } else {
+            RUN("argmax", (size_t)m->d.vocab_size * 4, k::argmax(s, row, UZU_F32, st->d_out_token, m->d.vocab_size, 1, m->argmax_scratch));
+        }
+    }
+    if (e.st != UZU_OK) return e.st;
+    hipLaunchKernelGGL(s32_commit_kernel, dim3(1), dim3(1), 0, s, st->d_ctx_len, st->d_tokens, st->d_out_token, st->d_sampled, count, sample ? 1u : 0u);
+    ++m->launches;
+    return UZU_OK;
+}
+
+} // namespace
+
+// ---------------------------------------------------------------------------------- construction
+
+uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t flags, uzu_hip_model** out) {
+    const uint32_t d = desc->model_dim, nl = desc->num_layers;
+    UZU_REQUIRE(desc->tied_embeddings && desc->embedding.method == UZU_QUANT_NONE && desc->embedding.weights && desc->embedding.n == desc->vocab_size && desc->embedding.k == d,
+                "model_create: an f32-stream design reads out through its full-precision embedding table [vocab, model_dim]");
+    UZU_REQUIRE(desc->output_norm.present && desc->output_norm.kind == UZU_NORM_DYNAMIC_TANH && desc->output_norm.scales, "model_create: an f32-stream design ends in a dynamic-tanh norm");
+    UZU_UNSUPPORTED(desc->has_ple || desc->embedding_norm.present || desc->num_ropes || desc->logit_soft_cap != 0.0f || desc->logit_scale != 1.0f || desc->input_scale != 1.0f,
+                    "model_create: decoder options of the bf16-stream families on an f32-stream design");
+    auto full = [](const uzu_linear_desc& L, uint32_t n, uint32_t kk) { return L.weights && L.method == UZU_QUANT_NONE && L.n == n && L.k == kk && !L.input_signs && !L.output_signs && !L.lora_rank; };
+    for (uint32_t l = 0; l < nl; ++l) {
+        const uzu_layer_desc& h = desc->layers[l];
+        UZU_UNSUPPORTED(h.mixer_kind != UZU_MIXER_LATENT_ATTENTION, "model_create: layer %u: an f32-stream design's mixer is latent attention", l);
+        UZU_REQUIRE(h.pre_mixer_norm.present && h.pre_mixer_norm.kind == UZU_NORM_DYNAMIC_TANH && h.pre_mixer_norm.scales, "model_create: layer %u needs a dynamic-tanh pre-mixer norm", l);
+        UZU_REQUIRE(h.num_heads && h.head_dim && h.value_head_dim && h.latent_rank && h.latent_rank <= k::kLatentMaxRank, "model_create: layer %u: heads / head_dim / value_head_dim / latent_rank (<= %u)",
+                    l, k::kLatentMaxRank);
+        UZU_REQUIRE(full(h.qkv_projection, h.num_heads * h.head_dim, d) && full(h.out_projection, d, h.num_heads * h.value_head_dim) &&
+                    full(h.latent_up_keys, h.num_heads * h.head_dim, h.latent_rank) && full(h.latent_up_values, h.num_heads * h.value_head_dim, h.latent_rank),
+                    "model_create: layer %u: query / out / latent up projections must be full-precision matrices of the configured shapes", l);
+        if (h.is_kv_sharing) {
+            UZU_REQUIRE(h.kv_source_layer_index < l, "model_create: layer %u shares the latents of layer %u, which does not precede it", l, h.kv_source_layer_index);
+            const uzu_layer_desc& src = desc->layers[h.kv_source_layer_index];
+            UZU_REQUIRE(!src.is_kv_sharing && src.latent_rank == h.latent_rank, "model_create: layer %u: the source layer %u must own latents of the same rank", l, h.kv_source_layer_index);
+        } else {
+            UZU_REQUIRE(full(h.latent_down, h.latent_rank, d) && h.latent_norm.present && h.latent_norm.scales, "model_create: layer %u owns its latents: down projection + latent norm required", l);
+        }
+        UZU_REQUIRE(!h.has_sinks || h.sinks, "model_create: layer %u: has_sinks without the tensor", l);
+        UZU_REQUIRE(!h.depth_weights || h.num_depth_weights == l + 2, "model_create: layer %u: a depth mix takes %u weights", l, l + 2);
+        if (!h.no_mlp) {
+            UZU_REQUIRE(h.pre_mlp_norm.present && h.pre_mlp_norm.kind == UZU_NORM_DYNAMIC_TANH && h.pre_mlp_norm.scales, "model_create: layer %u needs a dynamic-tanh pre-MLP norm", l);
+            if (h.mlp_kind == UZU_MLP_MOE) {
+                const uzu_moe_desc& M = h.moe;
+                UZU_REQUIRE(M.routing == UZU_MOE_ROUTE_SCORES && M.num_active_experts && M.num_active_experts <= M.num_routed_experts + M.num_identity_experts && M.router_weights &&
+                            (M.num_routed_experts == 0 || (M.expert_hidden_dim && M.w13 && M.w2)) && M.gating_sel == 2,
+                            "model_create: layer %u: score-routed SiLU-gated experts with their router and expert tensors", l);
+            } else {
+                UZU_REQUIRE(h.mlp_plain && h.activation == UZU_ACT_RELU_SQUARED && full(h.up_projection, h.hidden_dim, d) && full(h.down_projection, d, h.hidden_dim),
+                            "model_create: layer %u: the dense block is down(relu(up x + b)^2) + b with full-precision matrices", l);
+            }
+        }
+    }
+    (void)hipSetDevice(ctx->device);
+    auto* m = new uzu_hip_model();
+    m->ctx = ctx, m->flags = flags, m->d = *desc;
+    m->d.layers = nullptr;
+    auto* Sp = new Stream32();
+    m->s32 = Sp;
+    Stream32& S = *Sp;
+    S.full_f32 = (flags & UZU_MODEL_FULL_F32) != 0;
+    uzu_status st = UZU_OK;
+    auto fail = [&](uzu_status r) {
+        uzu_hip_model_destroy(m);
+        return r;
+    };
+#define TRY(x) do { st = (x); if (st != UZU_OK) return fail(st); } while (0)
+    TRY(upload_linear(m, desc->embedding, &m->embedding, true));
+    TRY(upload_norm(m, desc->output_norm, d, &m->output_norm));
+    S.alpha_out = desc->output_norm.alpha;
+    m->chunk = prefill_chunk_rows();
+    m->max_positions = desc->max_context_length + m->chunk;
+    m->max_seqs = (flags >> 8) & 0xFF ? (flags >> 8) & 0xFF : 1;
+    S.max_rows = m->chunk, S.max_seqs = m->max_seqs;
+    m->layers.resize(nl);
+    S.layers.resize(nl);
+    uint32_t w_q = 0, w_rank = 0, w_lat = 0, w_attn = 0, w_hid = 0, w_top = 1;
+    for (uint32_t l = 0; l < nl; ++l) {
+        const uzu_layer_desc& h = desc->layers[l];
+        DLayer& L = m->layers[l];
+        Stream32::Layer& X = S.layers[l];
+        L.d = h;
+        L.last_reader = l;
+        TRY(upload_norm(m, h.pre_mixer_norm, d, &L.pre_mixer));
+        X.alpha1 = h.pre_mixer_norm.alpha;
+        TRY(upload_linear(m, h.qkv_projection, &L.qkv));
+        TRY(upload_linear(m, h.out_projection, &L.out));
+        TRY(upload_linear(m, h.latent_up_values, &L.lat_up_v));
+        {   // W_up_k [heads * head_dim, rank] -> per head [rank, head_dim] (bf16 bits move, nothing is rounded)
+            const uint32_t H = h.num_heads, hd = h.head_dim, rank = h.latent_rank;
+            const uint16_t* src = (const uint16_t*)h.latent_up_keys.weights;
+            std::vector<uint16_t> t((size_t)H * rank * hd);
+            for (uint32_t hh = 0; hh < H; ++hh)
+                for (uint32_t i = 0; i < hd; ++i)
+                    for (uint32_t c = 0; c < rank; ++c) t[((size_t)hh * rank + c) * hd + i] = src[((size_t)hh * hd + i) * rank + c];
+            TRY(upload(m, t.data(), t.size() * 2, &X.up_keys_t));
+        }
+        if (!h.is_kv_sharing) {
+            TRY(upload_linear(m, h.latent_down, &L.lat_down));
+            TRY(upload_norm(m, h.latent_norm, h.latent_rank, &L.lat_norm));
+        }
+        if (h.has_sinks) {
+            std::vector<float> f(h.num_heads);
+            for (uint32_t i = 0; i < h.num_heads; ++i) f[i] = bf16_to_f32(((const uint16_t*)h.sinks)[i]);
+            TRY(upload(m, f.data(), f.size() * 4, &X.sinks));
+        }
+        if (h.token_shift) TRY(upload(m, h.token_shift, (size_t)d * 4, &X.token_shift));
+        if (h.depth_weights) TRY(upload(m, h.depth_weights, (size_t)h.num_depth_weights * 4, &X.depth_weights));
+        if (!h.no_mlp) {
+            TRY(upload_norm(m, h.pre_mlp_norm, d, &L.pre_mlp));
+            X.alpha2 = h.pre_mlp_norm.alpha;
+            if (h.mlp_kind == UZU_MLP_MOE) {
+                const uzu_moe_desc& M = h.moe;
+                const size_t E = M.num_routed_experts, ff = M.expert_hidden_dim;
+                TRY(upload(m, M.router_weights, (E + M.num_identity_experts) * d * 2, &L.moe.router_weights));
+                if (E) {
+                    TRY(upload(m, M.w13, E * 2 * ff * d * 2, &L.moe.w13));
+                    TRY(upload(m, M.w2, E * d * ff * 2, &L.moe.w2));
+                }
+                if (M.selection_bias) TRY(upload(m, M.selection_bias, (E + M.num_identity_experts) * 4, &X.selection_bias));
+                w_hid = std::max<uint32_t>(w_hid, M.num_active_experts * M.expert_hidden_dim);
+                w_top = std::max(w_top, M.num_active_experts);
+            } else {
+                TRY(upload_linear(m, h.up_projection, &L.up));
+                TRY(upload_linear(m, h.down_projection, &L.down));
+                w_hid = std::max(w_hid, h.hidden_dim);
+            }
+        }
+        w_q = std::max(w_q, h.num_heads * h.head_dim), w_rank = std::max(w_rank, h.latent_rank), w_lat = std::max(w_lat, h.num_heads * h.latent_rank);
+        w_attn = std::max(w_attn, h.num_heads * h.value_head_dim);
+    }
+    const size_t R = S.max_rows;
+    TRY(need_f32(m, (size_t)(nl + 1) * R * d, &S.slots));
+    TRY(need_f32(m, R * d, &S.xin));
+    TRY(need_f32(m, R * d, &S.normed));
+    TRY(need_f32(m, R * d, &S.out_normed));
+    TRY(need_f32(m, R * w_q, &S.q));
+    TRY(need_f32(m, R * w_rank, &S.ckv));
+    TRY(need_f32(m, R * w_lat, &S.qlat));
+    TRY(need_f32(m, R * w_lat, &S.ctx));
+    TRY(need_f32(m, R * w_attn, &S.attn));
+    TRY(need_f32(m, R * (w_hid ? w_hid : 1), &S.hid));
+    TRY(need_f32(m, R * w_top, &S.moe_w));
+    void* p = nullptr;
+    TRY(dev_alloc(m, R * w_top * 4, &p, true)); S.moe_ids = (int32_t*)p;
+    TRY(dev_alloc(m, S.max_seqs * sizeof(k::SeqSpan), &p, true)); S.d_spans = (k::SeqSpan*)p;
+    TRY(dev_alloc(m, R * 4, &p, true)); S.d_row_seq = (uint32_t*)p;
+    TRY(dev_alloc(m, R * 4, &p, true)); S.d_out_rows = (uint32_t*)p;
+    TRY(dev_alloc(m, (size_t)nl * S.max_seqs * sizeof(void*), &p, true)); S.d_cache_ptrs = (void**)p;
+    TRY(dev_alloc(m, (size_t)nl * S.max_seqs * sizeof(float*), &p, true)); S.d_shift_ptrs = (float**)p;
+    TRY(dev_alloc(m, R * 4, &p, true)); m->batch_tokens = (uint32_t*)p;
+    if (flags & UZU_MODEL_DEBUG_TAPS) TRY(need_f32(m, (size_t)nl * R * d, &S.taps));
+    TRY(dev_alloc(m, k::argmax_scratch_bytes(1), &m->argmax_scratch));
+    TRY(dev_alloc(m, k::unified_sampling_scratch_bytes(1), &m->sampling_scratch));
+    TRY(dev_alloc(m, 8, &p, true)); m->d_seed = (uint64_t*)p;
+    TRY(ensure_logits(m, 16));
+    TRY(state_build(m, &m->state0));
+    bind_state(m, m->state0);
+    if (hipEventCreate(&m->ev0) != hipSuccess || hipEventCreate(&m->ev1) != hipSuccess) {
+        set_error("model_create: hipEventCreate failed");
+        return fail(UZU_ERR_HIP);
+    }
+    if (hipStreamSynchronize(ctx->stream) != hipSuccess) {
+        set_error("model_create: synchronising the uploads failed");
+        return fail(UZU_ERR_HIP);
+    }
+#undef TRY
+    *out = m;
+    return UZU_OK;
+}
+
+void s32_destroy(uzu_hip_model* m) {
+    delete m->s32;
+    m->s32 = nullptr;
+}
+
+// the state rows of one layer (state_build, engine_build.hip): the latent cache of a layer that owns one, the token shift's last row
+uzu_status s32_state_layer(uzu_hip_model* m, uzu_hip_state* st, uint32_t l) {
+    const uzu_layer_desc& h = m->layers[l].d;
+    void* p = nullptr;
+    if (!h.is_kv_sharing) { // rows are written before they are read (latent_norm_append precedes the core in every pass)
+        UZU_PROPAGATE(state_alloc(st, (size_t)m->max_positions * h.latent_rank * (m->s32->full_f32 ? 4 : 2), &p, false));
+        st->layers[l].latent = p;
+    }
+    if (h.token_shift) {
+        UZU_PROPAGATE(state_alloc(st, (size_t)m->d.model_dim * 4, &p));
+        st->layers[l].shift_prev = (float*)p;
+    }
+    return UZU_OK;
+}
+
+// ---------------------------------------------------------------------------------- the C ABI's f32-stream legs (engine_api.hip dispatches here)
+
+// A batched step: sequence i appends counts[i] tokens.  want_rows index the concatenated token list; their logits go to logits_out [nwant][vocab] (host, f32).
+// sampled_out (optional) [nseq]: the token sampled from every sequence's last row (greedy; the model's stochastic sampler when one sequence is stepped); the
+// sampled token also becomes the sequence's next input token (uzu_hip_model_decode continues from it).
+uzu_status s32_step_batch(uzu_hip_model* m, uzu_hip_state** states, uint32_t nseq, const uint32_t* token_ids, const uint32_t* counts, const uint32_t* want_rows, uint32_t nwant,
+                          float* logits_out, uint32_t* sampled_out) {
+    Stream32& S = *m->s32;
+    hipStream_t s = m->ctx->stream;
+    const uint32_t V = m->d.vocab_size;
+    std::vector<uint32_t> offset(nseq + 1, 0), done(nseq, 0);
+    for (uint32_t i = 0; i < nseq; ++i) {
+        UZU_REQUIRE(states[i] && states[i]->m == m, "model_step_batch: state %u is null or belongs to another model", i);
+        for (uint32_t j = 0; j < i; ++j) UZU_REQUIRE(states[i] != states[j], "model_step_batch: state %u listed twice", i);
+        UZU_REQUIRE(counts[i] > 0, "model_step_batch: sequence %u brings no token", i);
+        UZU_REQUIRE(state_length(m, states[i]) + counts[i] <= m->d.max_context_length, "model_step_batch: sequence %u exceeds max_context_length %u", i, m->d.max_context_length);
+        offset[i + 1] = offset[i] + counts[i];
+    }
+    const uint32_t total = offset[nseq];
+    for (uint32_t i = 0; i < total; ++i) UZU_REQUIRE(token_ids[i] < V, "model_step_batch: token id %u outside the vocabulary", token_ids[i]);
+    for (uint32_t i = 0; i < nwant; ++i) UZU_REQUIRE(want_rows[i] < total && (i == 0 || want_rows[i] > want_rows[i - 1]), "model_step_batch: want_rows must be ascending rows of the step");
+    UZU_REQUIRE(!nwant || logits_out, "model_step_batch: logits wanted without a buffer");
+    const bool sample = sampled_out != nullptr;
+    uint32_t seq_lo = 0;
+    // passes: at most max_seqs sequences and max_rows rows each, sequences in order, a long prompt continues in the next pass
+    while (seq_lo < nseq) {
+        std::vector<PassSeq> pass;
+        std::vector<uint32_t> pass_tok, out_rows, out_dst, sample_seq;
+        uint32_t rows = 0, i = seq_lo;
+        for (; i < nseq && pass.size() < S.max_seqs && rows < S.max_rows; ++i) {
+            const uint32_t take = std::min(counts[i] - done[i], S.max_rows - rows);
+            const uint32_t first = offset[i] + done[i];
+            pass.push_back({states[i], take, state_length(m, states[i])});
+            for (uint32_t j = 0; j < take; ++j) pass_tok.push_back(token_ids[first + j]);
+            // wanted rows inside [first, first + take)
+            const uint32_t* lo = std::lower_bound(want_rows, want_rows + nwant, first);
+            for (const uint32_t* w = lo; w < want_rows + nwant && *w < first + take; ++w) out_rows.push_back(rows + (*w - first)), out_dst.push_back((uint32_t)(w - want_rows));
+            rows += take;
+            done[i] += take;
+            if (done[i] < counts[i]) break; // the rest of this prompt opens the next pass
+        }
+        for (size_t a = 0; a < pass.size(); ++a) {
+            const uint32_t qi = seq_lo + (uint32_t)a;
+            if (sample && done[qi] == counts[qi]) sample_seq.push_back((uint32_t)a);
+        }
+        const size_t n_want_rows = out_rows.size();
+        {
+            uint32_t r0 = 0;
+            std::vector<uint32_t> last_row(pass.size());
+            for (size_t a = 0; a < pass.size(); ++a) r0 += pass[a].count, last_row[a] = r0 - 1;
+            for (uint32_t a : sample_seq) out_rows.push_back(last_row[a]);
+        }
+        UZU_PROPAGATE(ensure_logits(m, out_rows.size()));
+        HIPCHK(hipMemcpyAsync(m->batch_tokens, pass_tok.data(), pass_tok.size() * 4, hipMemcpyHostToDevice, s));
+        UZU_PROPAGATE(s32_pass(m, pass, m->batch_tokens, out_rows));
+        for (size_t a = 0; a < pass.size(); ++a) {
+            const uint32_t qi = seq_lo + (uint32_t)a;
+            const bool finished = done[qi] == counts[qi];
+            size_t srow = 0;
+            bool do_sample = false;
+            for (size_t b = 0; b < sample_seq.size(); ++b)
+                if (sample_seq[b] == a) srow = n_want_rows + b, do_sample = true;
+            (void)finished;
+            UZU_PROPAGATE(sample_commit(m, pass[a].st, (uint32_t)srow, pass[a].count, do_sample));
+        }
+        HIPCHK(hipStreamSynchronize(s));
+        for (size_t a = 0; a < pass.size(); ++a) state_set_length(m, pass[a].st, pass[a].start + pass[a].count);
+        for (size_t b = 0; b < n_want_rows; ++b)
+            HIPCHK(hipMemcpy(logits_out + (size_t)out_dst[b] * V, S.logits + b * V, (size_t)V * 4, hipMemcpyDeviceToHost));
+        for (size_t b = 0; b < sample_seq.size(); ++b) {
+            const uint32_t qi = seq_lo + sample_seq[b];
+            HIPCHK(hipMemcpy(sampled_out + qi, states[qi]->d_out_token, 4, hipMemcpyDeviceToHost));
+        }
+        // sequences that are through leave the window; one that is not stays first
+        while (seq_lo < nseq && done[seq_lo] == counts[seq_lo]) ++seq_lo;
+    }
+    m->hidden_ready = false;
+    return UZU_OK;
+}
+
+uzu_status s32_prefill(uzu_hip_model* m, const uint32_t* token_ids, uint32_t count, uint32_t* first_token) {
+    uzu_hip_state* st = m->bound;
+    uint32_t sampled = 0;
+    UZU_PROPAGATE(s32_step_batch(m, &st, 1, token_ids, &count, nullptr, 0, nullptr, &sampled));
+    if (first_token) *first_token = sampled;
+    return UZU_OK;
+}
+
+// `steps` chained decode steps of the bound sequence: the input token of a step is the one the step before left in the control block
+uzu_status s32_decode_enqueue(uzu_hip_model* m, uint32_t steps) {
+    uzu_hip_state* st = m->bound;
+    UZU_REQUIRE(m->context_length + steps <= m->d.max_context_length, "model_decode: %u + %u tokens exceed max_context_length %u", m->context_length, steps, m->d.max_context_length);
+    UZU_PROPAGATE(ensure_logits(m, 1));
+    const std::vector<uint32_t> out_rows{0};
+    for (uint32_t i = 0; i < steps; ++i) {
+        const std::vector<PassSeq> pass{{st, 1, m->context_length}};
+        UZU_PROPAGATE(s32_pass(m, pass, st->d_tokens, out_rows));
+        UZU_PROPAGATE(sample_commit(m, st, 0, 1, true));
+        state_set_length(m, st, m->context_length + 1);
+    }
+    return UZU_OK;
+}
+
+uzu_status s32_read_logits_f32(uzu_hip_model* m, float* out, uint32_t row) {
+    Stream32& S = *m->s32;
+    UZU_REQUIRE(row < S.last_logit_rows, "model_read_logits: the last pass produced %u rows of logits", S.last_logit_rows);
+    HIPCHK(hipStreamSynchronize(m->ctx->stream));
+    HIPCHK(hipMemcpy(out, S.logits + (size_t)row * m->d.vocab_size, (size_t)m->d.vocab_size * 4, hipMemcpyDeviceToHost));
+    return UZU_OK;
+}
+
+uint32_t s32_last_logit_rows(const uzu_hip_model* m) { return m->s32->last_logit_rows; }
+
+uzu_status s32_read_layer_output(uzu_hip_model* m, uint32_t layer, float* out, uint32_t* rows) {
+    Stream32& S = *m->s32;
+    UZU_REQUIRE(S.taps, "model_read_layer_output: create the model with UZU_MODEL_DEBUG_TAPS");
+    UZU_REQUIRE(layer < m->d.num_layers, "model_read_layer_output: layer out of range");
+    HIPCHK(hipStreamSynchronize(m->ctx->stream));
+    if (rows) *rows = S.tap_rows;
+    if (out) HIPCHK(hipMemcpy(out, S.taps + (size_t)layer * S.max_rows * m->d.model_dim, (size_t)S.tap_rows * m->d.model_dim * 4, hipMemcpyDeviceToHost));
+    return UZU_OK;
+}
+
+} // namespace eng
+} // namespace uzu

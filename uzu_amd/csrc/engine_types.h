@@ -20,6 +20,7 @@ struct uzu_hip_state;
 
 namespace uzu {
 namespace eng {
+struct Stream32; // engine_stream32.hip: scratch, tables and per-layer extras of an f32-stream design
 
 constexpr uint32_t kSuffixCapacity = 1024; // ATTENTION_SUFFIX_CAPACITY, mixer/attention/state.rs:14: the reference's rows per forward pass (and its single- / two-pass rule)
 // Rows of one PREFILL pass here (uzu_hip_model::chunk; UZU_PREFILL_CHUNK = 1024 ... 8192, a multiple of 1024).  The reference feeds a prompt in
@@ -63,6 +64,10 @@ struct DLayer {
     uzu_layer_desc d; // scalars only (pointers are host pointers: never dereferenced after create)
     DNorm pre_mixer, post_mixer, pre_mlp, post_mlp, qn, kn;
     DLinear qkv, gate, out, in_proj, out_proj, up, down;
+    // latent attention (UZU_MIXER_LATENT_ATTENTION; engine_stream32.hip): down projection + RMS norm of the latent, value up projection (the key up projection
+    // lives transposed per head in Stream32::Layer)
+    DLinear lat_down, lat_up_v;
+    DNorm lat_norm;
     float *conv_w = nullptr, *conv_b = nullptr, *a_log = nullptr, *dt_bias = nullptr, *dn_norm = nullptr;
     uint16_t* sinks = nullptr; // bf16 [heads] (has_sinks)
     // the layer's RoPE configuration (uzu_model_desc::ropes[rope_index], or the model's single `rope`): tables [max positions][rope_dim]
@@ -83,6 +88,19 @@ struct DLayer {
     } moe;
 };
 
+
+// ---- engine_stream32.hip: the f32-stream designs (uzu_model_desc::f32_stream)
+uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t flags, uzu_hip_model** out);
+void s32_destroy(uzu_hip_model* m);
+uzu_status s32_state_layer(uzu_hip_model* m, uzu_hip_state* st, uint32_t layer);
+uzu_status s32_step_batch(uzu_hip_model* m, uzu_hip_state** states, uint32_t nseq, const uint32_t* token_ids, const uint32_t* counts, const uint32_t* want_rows, uint32_t nwant,
+                          float* logits_out, uint32_t* sampled_out);
+uzu_status s32_prefill(uzu_hip_model* m, const uint32_t* token_ids, uint32_t count, uint32_t* first_token);
+uzu_status s32_decode_enqueue(uzu_hip_model* m, uint32_t steps);
+uzu_status s32_read_logits_f32(uzu_hip_model* m, float* out, uint32_t row);
+uint32_t s32_last_logit_rows(const uzu_hip_model* m);
+uzu_status s32_read_layer_output(uzu_hip_model* m, uint32_t layer, float* out, uint32_t* rows);
+
 } // namespace eng
 } // namespace uzu
 
@@ -101,6 +119,9 @@ struct uzu_hip_state {
     struct Layer {
         uint16_t *keys = nullptr, *values = nullptr;
         float *conv_state = nullptr, *ssm_state = nullptr;
+        // f32-stream designs: the latent cache of a layer that owns one ([max positions][latent_rank], bf16 or f32) and the token shift's last normalised row
+        void* latent = nullptr;
+        float* shift_prev = nullptr;
     };
     std::vector<Layer> layers;
     uint32_t *d_ctx_len = nullptr, *d_tokens = nullptr, *d_out_token = nullptr, *d_sampled = nullptr;
@@ -275,6 +296,7 @@ struct uzu_hip_model {
     uint32_t final_hidden_rows = 0;
     void* prof_sink = nullptr; // std::vector<ProfEntry>* while profiling one step
     int regime_override = -1; // graph capture: 0 = single-pass attention, 1 = two-pass (else decided by context_length)
+    uzu::eng::Stream32* s32 = nullptr; // non-null: an f32-stream design; prefill / decode / batched steps run through engine_stream32.hip
 };
 
 namespace uzu {

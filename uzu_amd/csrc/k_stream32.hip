@@ -1,0 +1,381 @@
+// k_stream32.hip -- element-wise kernels, the full-precision linear and the score-routed experts of the f32-stream designs (kernels_stream32.h).
+//
+// Everything here keeps f32 where such a design asks for it: the residual rows, the norm, the router and its softmax, every accumulation.  A matrix product
+// reads f32 activation rows and bf16 weights; with `bf16_products` the activation operand is rounded to bf16 as it is loaded (what a bf16 activation buffer
+// would have held), otherwise the product is a true f32 product.  Reductions run in a fixed order: a result does not depend on what else is in the pass.
+#include "device_utils.h"
+#include "kernels_stream32.h"
+
+namespace uzu {
+namespace k {
+
+namespace {
+
+__device__ __forceinline__ float opnd(float v, uint32_t bf16_products) { return bf16_products ? round_bf16(v) : v; }
+
+__global__ void __launch_bounds__(256) embed_rows_f32_kernel(const uint32_t* tokens, const uint16_t* table, float* out, uint32_t vocab, uint32_t d) {
+    const uint32_t r = blockIdx.x;
+    uint32_t t = tokens[r];
+    if (t >= vocab) t = 0;
+    const uint16_t* src = table + (size_t)t * d;
+    float* dst = out + (size_t)r * d;
+    for (uint32_t i = threadIdx.x; i < d; i += blockDim.x) dst[i] = bf16_to_f32(src[i]);
+}
+
+__global__ void __launch_bounds__(256) dyn_tanh_kernel(DynTanhParams p) {
+    const uint32_t r = blockIdx.x;
+    const uint32_t src = p.row_index ? p.row_index[r] : r;
+    const float* x = p.x + (size_t)src * p.d;
+    float* out = p.out + (size_t)r * p.d;
+    if (!p.shift) {
+        for (uint32_t i = threadIdx.x; i < p.d; i += blockDim.x) out[i] = fmaf(tanhf(p.alpha * x[i]), p.scales[i], p.biases ? p.biases[i] : 0.0f);
+        return;
+    }
+    const uint32_t q = p.row_seq[r];
+    const SeqSpan sp = p.spans[q];
+    const bool first = r == sp.row0;
+    float* prev = p.prev[q];
+    const float* xl = p.x + (size_t)(sp.row0 + sp.count - 1) * p.d; // the sequence's last row of the pass
+    for (uint32_t i = threadIdx.x; i < p.d; i += blockDim.x) {
+        const float w = p.scales[i], b = p.biases ? p.biases[i] : 0.0f;
+        const float h = fmaf(tanhf(p.alpha * x[i]), w, b);
+        float hp;
+        if (first) {
+            hp = sp.start ? prev[i] : 0.0f;
+            // the same thread that has read the state's element replaces it: no other block of the launch touches prev[q]
+            prev[i] = sp.count == 1 ? h : fmaf(tanhf(p.alpha * xl[i]), w, b);
+        } else {
+            hp = fmaf(tanhf(p.alpha * x[(ptrdiff_t)i - (ptrdiff_t)p.d]), w, b);
+        }
+        out[i] = fmaf(hp - h, p.shift[i], h);
+    }
+}
+
+__global__ void __launch_bounds__(256) depth_mix_kernel(const float* slots, size_t slot_stride, const float* w, uint32_t count, float* out, size_t total) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    float acc = 0.0f;
+    for (uint32_t j = 0; j < count; ++j) acc = fmaf(w[j], slots[(size_t)j * slot_stride + i], acc);
+    out[i] = acc;
+}
+
+__device__ __forceinline__ float apply_act(float v, uint32_t act) {
+    if (act == 1) {
+        const float t = fmaxf(v, 0.0f);
+        return t * t;
+    }
+    return v;
+}
+
+// ---- few rows: a wave per output column, RT rows per pass over the weights
+template <int RT>
+__global__ void __launch_bounds__(256) linear_rows_kernel(LinearF32Params p, uint32_t vec) {
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t n = blockIdx.x * 4 + wave;
+    const uint32_t r0 = blockIdx.y * RT;
+    const uint32_t z = blockIdx.z;
+    if (n >= p.n) return;
+    const float* x = p.x + z * p.x_batch;
+    const uint16_t* w = p.w + z * p.w_batch + (size_t)n * p.k;
+    float acc[RT];
+#pragma unroll
+    for (int i = 0; i < RT; ++i) acc[i] = 0.0f;
+    if (vec) {
+        for (uint32_t k0 = lane * 8; k0 < p.k; k0 += 64 * 8) {
+            const uint4 wv = *(const uint4*)(w + k0);
+            const uint32_t ww[4] = {wv.x, wv.y, wv.z, wv.w};
+            float wf[8];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) wf[2 * j] = bits_to_f32(ww[j] << 16), wf[2 * j + 1] = bits_to_f32(ww[j] & 0xFFFF0000u);
+#pragma unroll
+            for (int i = 0; i < RT; ++i) {
+                const uint32_t r = r0 + i < p.rows ? r0 + i : p.rows - 1;
+                const float4 a = *(const float4*)(x + (size_t)r * p.ldx + k0), b = *(const float4*)(x + (size_t)r * p.ldx + k0 + 4);
+                const float xv[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc[i] = fmaf(opnd(xv[j], p.bf16_products), wf[j], acc[i]);
+            }
+        }
+    } else {
+        for (uint32_t k0 = lane; k0 < p.k; k0 += 64) {
+            const float wf = bf16_to_f32(w[k0]);
+#pragma unroll
+            for (int i = 0; i < RT; ++i) {
+                const uint32_t r = r0 + i < p.rows ? r0 + i : p.rows - 1;
+                acc[i] = fmaf(opnd(x[(size_t)r * p.ldx + k0], p.bf16_products), wf, acc[i]);
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < RT; ++i) acc[i] = wave_sum(acc[i]);
+    if (lane == 0) {
+        const float bias = p.bias ? bf16_to_f32(p.bias[n]) : 0.0f;
+        float* y = p.y + z * p.y_batch;
+#pragma unroll
+        for (int i = 0; i < RT; ++i) {
+            const uint32_t r = r0 + i;
+            if (r >= p.rows) break;
+            float v = apply_act(acc[i] + bias, p.act);
+            if (p.residual) v += p.residual[(size_t)r * p.ldr + n];
+            y[(size_t)r * p.ldy + n] = v;
+        }
+    }
+}
+
+// ---- many rows without the matrix cores (true f32 products, and every shape the matrix-core form does not take): 64 x 64 tile, 16-deep k-steps through LDS,
+// a 4 x 4 block of outputs per thread
+constexpr int TM = 64, TN = 64, TK = 16;
+__global__ void __launch_bounds__(256) linear_tile_kernel(LinearF32Params p) {
+    __shared__ float s_a[TK][TM + 4];
+    __shared__ float s_b[TK][TN + 4];
+    const uint32_t z = blockIdx.z;
+    const float* x = p.x + z * p.x_batch;
+    const uint16_t* w = p.w + z * p.w_batch;
+    const uint32_t m0 = blockIdx.y * TM, n0 = blockIdx.x * TN;
+    const uint32_t tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+    float acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = 0.0f;
+    // loader mapping: thread -> (row / column tid >> 2 of the tile, k offsets (tid & 3) * 4 .. + 3)
+    const uint32_t lr = tid >> 2, lk = (tid & 3) * 4;
+    for (uint32_t k0 = 0; k0 < p.k; k0 += TK) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t kk = k0 + lk + j;
+            const uint32_t r = m0 + lr, n = n0 + lr;
+            s_a[lk + j][lr] = (r < p.rows && kk < p.k) ? opnd(x[(size_t)r * p.ldx + kk], p.bf16_products) : 0.0f;
+            s_b[lk + j][lr] = (n < p.n && kk < p.k) ? bf16_to_f32(w[(size_t)n * p.k + kk]) : 0.0f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < TK; ++kk) {
+            float a[4], b[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) a[i] = s_a[kk][ty * 4 + i], b[i] = s_b[kk][tx * 4 + i];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+    float* y = p.y + z * p.y_batch;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t r = m0 + ty * 4 + i;
+        if (r >= p.rows) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t n = n0 + tx * 4 + j;
+            if (n >= p.n) continue;
+            float v = apply_act(acc[i][j] + (p.bias ? bf16_to_f32(p.bias[n]) : 0.0f), p.act);
+            if (p.residual) v += p.residual[(size_t)r * p.ldr + n];
+            y[(size_t)r * p.ldy + n] = v;
+        }
+    }
+}
+
+// ---- score routing: one wave per row
+constexpr uint32_t kRouteMaxOutputs = 512; // 8 per lane
+__global__ void __launch_bounds__(64) moe_route_scores_kernel(const float* x, const uint16_t* router, const float* selection_bias, int32_t* ids, float* weights, uint32_t d,
+                                                              uint32_t outputs, uint32_t top) {
+    const uint32_t r = blockIdx.x, lane = threadIdx.x;
+    const float* xr = x + (size_t)r * d;
+    float z[8];
+    float zmax = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) z[j] = -INFINITY;
+    for (uint32_t e = 0; e < outputs; ++e) {
+        const uint16_t* w = router + (size_t)e * d;
+        float acc = 0.0f;
+        for (uint32_t i = lane; i < d; i += 64) acc = fmaf(xr[i], bf16_to_f32(w[i]), acc);
+        acc = wave_sum(acc);
+        if ((e & 63) == lane) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                if ((uint32_t)j == (e >> 6)) z[j] = acc;
+        }
+        zmax = fmaxf(zmax, acc);
+    }
+    float ex[8], sum = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const uint32_t e = j * 64 + lane;
+        ex[j] = e < outputs ? expf(z[j] - zmax) : 0.0f;
+        sum += ex[j];
+    }
+    sum = wave_sum(sum);
+    float score[8], choice[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const uint32_t e = j * 64 + lane;
+        score[j] = ex[j] / sum;
+        choice[j] = e < outputs ? score[j] + (selection_bias ? selection_bias[e] : 0.0f) : -INFINITY;
+    }
+    float wsum = 0.0f;
+    float my_w = 0.0f; // lane t keeps the t-th winner's score
+    int32_t my_id = 0;
+    for (uint32_t t = 0; t < top; ++t) {
+        float best = -INFINITY;
+        uint32_t best_e = 0xFFFFFFFFu;
+        float best_s = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const uint32_t e = j * 64 + lane;
+            if (e < outputs && (choice[j] > best || (choice[j] == best && e < best_e))) best = choice[j], best_e = e, best_s = score[j];
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const float ob = __shfl_xor(best, off, 64), os = __shfl_xor(best_s, off, 64);
+            const uint32_t oe = __shfl_xor(best_e, off, 64);
+            if (ob > best || (ob == best && oe < best_e)) best = ob, best_e = oe, best_s = os;
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            if ((uint32_t)j * 64 + lane == best_e) choice[j] = -INFINITY; // taken (a NaN row leaves best_e invalid: every lane then agrees on 0xFFFFFFFF)
+        wsum += best_s;
+        if ((t & 63) == lane && t < 64) my_w = best_s, my_id = (int32_t)best_e;
+        if (t >= 64 && lane == 0) { // more winners than lanes: written as they come
+            ids[(size_t)r * top + t] = (int32_t)best_e;
+            weights[(size_t)r * top + t] = best_s; // (normalised below only for the first 64; top <= 64 is checked on the host)
+        }
+    }
+    if (lane < top && lane < 64) {
+        ids[(size_t)r * top + lane] = my_id;
+        weights[(size_t)r * top + lane] = my_w / (wsum + 1e-20f);
+    }
+}
+
+// a workgroup per (row, slot): the row once into LDS, then a wave per hidden unit (gate and up rows of the unit in the same pass)
+__global__ void __launch_bounds__(256) moe_experts_gate_up_kernel(const float* x, const int32_t* ids, const uint16_t* w13, float* hidden, uint32_t d, uint32_t ff, uint32_t routed,
+                                                                  uint32_t top, uint32_t bf16_products) {
+    extern __shared__ float s_x[];
+    const uint32_t slot = blockIdx.x, r = slot / top;
+    const int32_t e = ids[slot];
+    if (e < 0 || (uint32_t)e >= routed) return; // an identity expert has no hidden row
+    for (uint32_t i = threadIdx.x; i < d; i += blockDim.x) s_x[i] = opnd(x[(size_t)r * d + i], bf16_products);
+    __syncthreads();
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    const uint16_t* base = w13 + (size_t)e * 2 * ff * d;
+    for (uint32_t f = blockIdx.y * nw + wave; f < ff; f += gridDim.y * nw) {
+        const uint16_t* wu = base + (size_t)f * d;
+        const uint16_t* wg = base + (size_t)(ff + f) * d;
+        float au = 0.0f, ag = 0.0f;
+        for (uint32_t i = lane; i < d; i += 64) {
+            const float xv = s_x[i];
+            au = fmaf(xv, bf16_to_f32(wu[i]), au);
+            ag = fmaf(xv, bf16_to_f32(wg[i]), ag);
+        }
+        au = wave_sum(au), ag = wave_sum(ag);
+        if (lane == 0) hidden[(size_t)slot * ff + f] = ag / (1.0f + expf(-ag)) * au;
+    }
+}
+
+// a workgroup per (row, block of outputs): the row's hidden rows into LDS, then a wave per output; the slots are added in slot order
+__global__ void __launch_bounds__(256) moe_experts_down_kernel(const float* hidden, const float* x, const int32_t* ids, const float* weights, const uint16_t* w2,
+                                                               const float* residual, float* y, uint32_t d, uint32_t ff, uint32_t routed, uint32_t top, uint32_t bf16_products) {
+    extern __shared__ float s_h[]; // [top][ff]
+    const uint32_t r = blockIdx.x;
+    for (uint32_t i = threadIdx.x; i < top * ff; i += blockDim.x) {
+        const int32_t e = ids[(size_t)r * top + i / ff];
+        s_h[i] = (e >= 0 && (uint32_t)e < routed) ? opnd(hidden[(size_t)r * top * ff + i], bf16_products) : 0.0f;
+    }
+    __syncthreads();
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    for (uint32_t n = blockIdx.y * nw + wave; n < d; n += gridDim.y * nw) {
+        float total = residual ? residual[(size_t)r * d + n] : 0.0f;
+        for (uint32_t j = 0; j < top; ++j) {
+            const int32_t e = ids[(size_t)r * top + j];
+            const float wt = weights[(size_t)r * top + j];
+            if (e < 0) continue;
+            if ((uint32_t)e >= routed) { // identity expert: the block's input itself
+                total = fmaf(wt, x[(size_t)r * d + n], total);
+                continue;
+            }
+            const uint16_t* w = w2 + ((size_t)e * d + n) * ff;
+            float acc = 0.0f;
+            for (uint32_t i = lane; i < ff; i += 64) acc = fmaf(s_h[j * ff + i], bf16_to_f32(w[i]), acc);
+            acc = wave_sum(acc);
+            total = fmaf(wt, acc, total);
+        }
+        if (lane == 0) y[(size_t)r * d + n] = total;
+    }
+}
+
+} // namespace
+
+uzu_status embed_rows_f32(hipStream_t s, const uint32_t* tokens, const uint16_t* table, float* out, uint32_t rows, uint32_t vocab, uint32_t d) {
+    if (!rows) return UZU_OK;
+    return launch_check([&] { hipLaunchKernelGGL(embed_rows_f32_kernel, dim3(rows), dim3(256), 0, s, tokens, table, out, vocab, d); }, "embed_rows_f32");
+}
+
+uzu_status dyn_tanh_norm(hipStream_t s, const DynTanhParams& p) {
+    if (!p.rows) return UZU_OK;
+    UZU_REQUIRE(p.x && p.out && p.scales, "dyn_tanh_norm: null argument");
+    UZU_REQUIRE(!p.shift || (p.spans && p.row_seq && p.prev && !p.row_index), "dyn_tanh_norm: the token shift needs the pass's spans, row map and state rows");
+    UZU_REQUIRE(!p.shift || p.x != p.out, "dyn_tanh_norm: the token shift reads neighbouring rows: not in place");
+    return launch_check([&] { hipLaunchKernelGGL(dyn_tanh_kernel, dim3(p.rows), dim3(256), 0, s, p); }, "dyn_tanh_norm");
+}
+
+uzu_status depth_mix(hipStream_t s, const float* slots, size_t slot_stride, const float* w, uint32_t count, float* out, uint32_t rows, uint32_t d) {
+    const size_t total = (size_t)rows * d;
+    if (!total) return UZU_OK;
+    return launch_check([&] { hipLaunchKernelGGL(depth_mix_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, s, slots, slot_stride, w, count, out, total); }, "depth_mix");
+}
+
+size_t linear_f32_bytes(const LinearF32Params& p) { return (size_t)p.batch * ((size_t)p.n * p.k * 2 + (size_t)p.rows * p.k * 4 + (size_t)p.rows * p.n * 4); }
+
+uzu_status linear_f32(hipStream_t s, const LinearF32Params& p, const char** variant) {
+    if (!p.rows || !p.n || !p.batch) return UZU_OK;
+    UZU_REQUIRE(p.x && p.w && p.y && p.k, "linear_f32: null argument");
+    UZU_REQUIRE(!p.residual || p.batch == 1, "linear_f32: a residual only with one product per launch");
+    UZU_REQUIRE(p.ldx >= p.k && p.ldy >= p.n && p.batch <= 65535, "linear_f32: row pitch below the row length");
+    if (p.rows <= 16) {
+        const uint32_t vec = (p.k % 8 == 0 && p.ldx % 4 == 0 && p.x_batch % 4 == 0 && p.w_batch % 8 == 0 && (uintptr_t)p.x % 16 == 0 && (uintptr_t)p.w % 16 == 0) ? 1u : 0u;
+        if (variant) *variant = "linear_rows";
+        if (p.rows <= 2) {
+            const dim3 grid((p.n + 3) / 4, (p.rows + 1) / 2, p.batch);
+            return launch_check([&] { hipLaunchKernelGGL(linear_rows_kernel<2>, grid, dim3(256), 0, s, p, vec); }, "linear_rows");
+        }
+        const dim3 grid((p.n + 3) / 4, (p.rows + 3) / 4, p.batch);
+        return launch_check([&] { hipLaunchKernelGGL(linear_rows_kernel<4>, grid, dim3(256), 0, s, p, vec); }, "linear_rows");
+    }
+    if (linear_mfma_supported(p)) {
+        if (variant) *variant = "linear_mfma";
+        return linear_mfma(s, p);
+    }
+    if (variant) *variant = "linear_tile";
+    const dim3 grid((p.n + TN - 1) / TN, (p.rows + TM - 1) / TM, p.batch);
+    UZU_REQUIRE(grid.y <= 65535, "linear_f32: too many rows for one launch");
+    return launch_check([&] { hipLaunchKernelGGL(linear_tile_kernel, grid, dim3(256), 0, s, p); }, "linear_tile");
+}
+
+uzu_status moe_route_scores(hipStream_t s, const float* x, const uint16_t* router, const float* selection_bias, int32_t* ids, float* weights, uint32_t rows, uint32_t d,
+                            uint32_t outputs, uint32_t top) {
+    if (!rows) return UZU_OK;
+    UZU_UNSUPPORTED(outputs > kRouteMaxOutputs || top > 64 || top > outputs || !top, "moe_route_scores: at most %u router outputs and 64 winners (got %u, %u)", kRouteMaxOutputs, outputs, top);
+    return launch_check([&] { hipLaunchKernelGGL(moe_route_scores_kernel, dim3(rows), dim3(64), 0, s, x, router, selection_bias, ids, weights, d, outputs, top); }, "moe_route_scores");
+}
+
+uzu_status moe_experts_gate_up(hipStream_t s, const float* x, const int32_t* ids, const uint16_t* w13, float* hidden, uint32_t rows, uint32_t d, uint32_t ff, uint32_t routed,
+                               uint32_t top, uint32_t bf16_products) {
+    if (!rows || !routed) return UZU_OK;
+    UZU_UNSUPPORTED((size_t)d * 4 > 64 * 1024, "moe_experts_gate_up: model_dim %u does not fit the workgroup's LDS row", d);
+    const uint32_t gy = ff >= 256 ? 4 : 1; // wide experts: several workgroups share a (row, slot)
+    return launch_check([&] { hipLaunchKernelGGL(moe_experts_gate_up_kernel, dim3(rows * top, gy), dim3(256), (size_t)d * 4, s, x, ids, w13, hidden, d, ff, routed, top, bf16_products); },
+                        "moe_experts_gate_up");
+}
+
+uzu_status moe_experts_down_combine(hipStream_t s, const float* hidden, const float* x, const int32_t* ids, const float* weights, const uint16_t* w2, const float* residual,
+                                    float* y, uint32_t rows, uint32_t d, uint32_t ff, uint32_t routed, uint32_t top, uint32_t bf16_products) {
+    if (!rows) return UZU_OK;
+    UZU_UNSUPPORTED((size_t)top * ff * 4 > 64 * 1024, "moe_experts_down_combine: %u slots x %u hidden units do not fit the workgroup's LDS", top, ff);
+    const uint32_t gy = d >= 1024 ? 4 : 1;
+    return launch_check([&] { hipLaunchKernelGGL(moe_experts_down_kernel, dim3(rows, gy), dim3(256), (size_t)top * ff * 4, s, hidden, x, ids, weights, w2, residual, y, d, ff, routed, top,
+                                                  bf16_products); }, "moe_experts_down_combine");
+}
+
+} // namespace k
+} // namespace uzu

@@ -1,0 +1,104 @@
+// kernels_stream32.h -- kernels of the f32-stream designs (uzu_model_desc::f32_stream): the residual stream, norms, attention scores / weights and routers
+// are f32; activations travel between kernels as f32 rows; weights are bf16 [n, k] in HBM.  `bf16_products` != 0: a matrix product rounds its activation
+// operand to bf16 (weights are bf16 already) and accumulates in f32 -- the serving precision; 0: every product is a true f32 product.
+//   k_stream32.hip           embedding rows, dynamic-tanh norm + token shift, depth mix, the full-precision linear, score-routed experts
+//   k_linear_mfma.hip        the full-precision linear on the matrix cores (bf16 products, prefill-sized row counts)
+//   k_latent_attention.hip   latent normalisation + cache append, the latent-space attention core (prompt rows and decode rows)
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/uzu_hip.h"
+
+namespace uzu {
+namespace k {
+
+// One sequence's share of a batched pass: its rows are row0 .. row0 + count - 1 of the pass, at positions start .. start + count - 1 of the sequence.
+struct SeqSpan {
+    uint32_t row0, count, start;
+};
+
+// out[r, :] = f32(table[token[r], :])   (table bf16 [vocab, d]; an id >= vocab reads row 0 and the host has refused it before)
+uzu_status embed_rows_f32(hipStream_t s, const uint32_t* tokens, const uint16_t* table, float* out, uint32_t rows, uint32_t vocab, uint32_t d);
+
+// Dynamic-tanh norm, optionally followed by the token shift:
+//   h[r]   = tanh(alpha * x[src(r)]) * scales + biases          src(r) = row_index ? row_index[r] : r
+//   out[r] = shift ? h[r] + (h[r - 1 of the same sequence] - h[r]) * shift : h[r]
+// The predecessor of a sequence's first row of the pass is prev[seq] (f32 [d], the state; zeros are used instead at position 0); the launch leaves the
+// sequence's last h there.  shift == nullptr: spans / row_seq / prev are unused.
+struct DynTanhParams {
+    const float* x;
+    float* out;
+    const float* scales;
+    const float* biases;
+    float alpha;
+    const float* shift;
+    const uint32_t* row_index;
+    const SeqSpan* spans;
+    const uint32_t* row_seq;
+    float* const* prev; // device array [nseq] of device pointers
+    uint32_t rows, d;
+};
+uzu_status dyn_tanh_norm(hipStream_t s, const DynTanhParams& p);
+
+// out[r, :] = sum_{j < count} w[j] * slots[j * slot_stride + r * d ...]
+uzu_status depth_mix(hipStream_t s, const float* slots, size_t slot_stride, const float* w, uint32_t count, float* out, uint32_t rows, uint32_t d);
+
+// Y[z][r, n] = act(sum_k X[z][r, k] * W[z][n, k] + bias[n]) + residual[r, n]        z < batch (grid.z): a batch of independent products of one shape
+//   X[z] = x + z * x_batch (row pitch ldx), W[z] = w + z * w_batch ([n, k] bf16), Y[z] = y + z * y_batch (row pitch ldy)
+//   act: 0 none, 1 max(.,0)^2.  residual (pitch ldr, only with batch == 1) may alias y.
+struct LinearF32Params {
+    const float* x;
+    const uint16_t* w;
+    const uint16_t* bias; // bf16 [n] or null
+    const float* residual;
+    float* y;
+    uint32_t rows, n, k;
+    uint32_t ldx, ldy, ldr;
+    uint32_t batch;
+    size_t x_batch, w_batch, y_batch; // element strides
+    uint32_t act;
+    uint32_t bf16_products;
+};
+uzu_status linear_f32(hipStream_t s, const LinearF32Params& p, const char** variant = nullptr);
+// the matrix-core form (k_linear_mfma.hip): bf16 products only; false = shape / mode not covered, nothing launched
+bool linear_mfma_supported(const LinearF32Params& p);
+uzu_status linear_mfma(hipStream_t s, const LinearF32Params& p);
+size_t linear_f32_bytes(const LinearF32Params& p);
+
+// Score routing: per row scores = softmax(router x) over all `outputs` (= routed + identity) in f32, the `top` largest (score + bias) win (ties: lower index),
+// weights = score / (sum of the winners' scores + 1e-20).  ids [rows, top] (>= routed: an identity expert), weights f32 [rows, top].
+uzu_status moe_route_scores(hipStream_t s, const float* x, const uint16_t* router, const float* selection_bias, int32_t* ids, float* weights, uint32_t rows, uint32_t d,
+                            uint32_t outputs, uint32_t top);
+// hidden[r * top + j, f] = silu(gate_e x_r) * (up_e x_r) for e = ids[r, j] < routed; w13 bf16 [routed][2 ff][d], rows [0, ff) of an expert = up, [ff, 2 ff) = gate
+uzu_status moe_experts_gate_up(hipStream_t s, const float* x, const int32_t* ids, const uint16_t* w13, float* hidden, uint32_t rows, uint32_t d, uint32_t ff, uint32_t routed,
+                               uint32_t top, uint32_t bf16_products);
+// y[r, :] = residual[r, :] + sum_j weights[r, j] * (ids[r, j] < routed ? down_e hidden[r * top + j] : x[r, :])   in slot order; w2 bf16 [routed][d][ff]; y may alias residual
+uzu_status moe_experts_down_combine(hipStream_t s, const float* hidden, const float* x, const int32_t* ids, const float* weights, const uint16_t* w2, const float* residual,
+                                    float* y, uint32_t rows, uint32_t d, uint32_t ff, uint32_t routed, uint32_t top, uint32_t bf16_products);
+
+// RMS norm of the latent rows (x / sqrt(mean(x^2) + eps) * scales) and append to the sequences' caches: row r goes to cache[seq(r)] + (position of r) * rank,
+// stored as bf16 (cache_bf16) or f32.
+uzu_status latent_norm_append(hipStream_t s, const float* x, const float* scales, float eps, void* const* caches, uint32_t cache_bf16, const SeqSpan* spans,
+                              const uint32_t* row_seq, uint32_t rows, uint32_t rank);
+
+// Latent-space attention core.  Row r (sequence q, position t) and head h: keys j = max(0, t - window + 1) .. t (window 0: from 0),
+//   s_j = scale * <qlat[r, h, :], c_j>,  weights = exp(s_j - m) / (sum_j exp(s_j - m) + exp(sink_h - m)),  out[r, h, :] = sum_j weights_j c_j
+// qlat / out f32 [rows, heads * rank]; c_j = caches[q][j * rank ...] (bf16 or f32); sinks f32 [heads] or null (no sink term).
+struct LatentAttentionParams {
+    const float* qlat;
+    float* out;
+    void* const* caches;
+    uint32_t cache_bf16;
+    const float* sinks;
+    const SeqSpan* spans;
+    const uint32_t* row_seq;
+    uint32_t rows, heads, rank, window;
+    float scale;
+};
+uzu_status latent_attention(hipStream_t s, const LatentAttentionParams& p);
+constexpr uint32_t kLatentMaxRank = 1024;
+
+} // namespace k
+} // namespace uzu

@@ -17,8 +17,10 @@ import numpy as np
 
 # enums (uzu_model_desc.h)
 QUANT_SCALE_BIAS, QUANT_SCALE_ZERO_POINT, QUANT_SCALE_SYMMETRIC, QUANT_NONE = 0, 1, 2, 3
-ACT_SILU, ACT_GELU_APPROX, ACT_GELU_EXACT, ACT_IDENTITY, ACT_SOFTPLUS = 0, 1, 2, 3, 4
-MIXER_ATTENTION, MIXER_DELTA_NET = 0, 1
+ACT_SILU, ACT_GELU_APPROX, ACT_GELU_EXACT, ACT_IDENTITY, ACT_SOFTPLUS, ACT_RELU_SQUARED = 0, 1, 2, 3, 4, 5
+MIXER_ATTENTION, MIXER_DELTA_NET, MIXER_LATENT_ATTENTION = 0, 1, 2
+NORM_STATISTICS, NORM_DYNAMIC_TANH = 0, 1
+MOE_ROUTE_TOPK_LOGITS, MOE_ROUTE_SCORES = 0, 1
 ROPE_NONE, ROPE_UNSCALED, ROPE_LLAMA, ROPE_LINEAR, ROPE_YARN, ROPE_LONGROPE = 0, 1, 2, 3, 4, 5
 
 
@@ -35,9 +37,10 @@ class LinearDesc(C.Structure):
 
 class NormDesc(C.Structure):
     _fields_ = [
-        ("present", C.c_uint32), ("full_layer", C.c_uint32), ("subtract_mean", C.c_uint32), ("reserved", C.c_uint32),
+        ("present", C.c_uint32), ("full_layer", C.c_uint32), ("subtract_mean", C.c_uint32), ("kind", C.c_uint32),
         ("epsilon", C.c_float), ("scale_offset", C.c_float),
         ("scales", C.c_void_p), ("biases", C.c_void_p),
+        ("alpha", C.c_float), ("reserved", C.c_uint32),
     ]
 
 
@@ -59,6 +62,7 @@ class MoeDesc(C.Structure):
         ("gating_sel", C.c_uint32), ("silu_alpha", C.c_float),
         ("gate_clip_min", C.c_float), ("gate_clip_max", C.c_float), ("up_clip_min", C.c_float), ("up_clip_max", C.c_float),
         ("router_weights", C.c_void_p), ("router_biases", C.c_void_p), ("w13", C.c_void_p), ("w2", C.c_void_p), ("up_biases", C.c_void_p), ("down_biases", C.c_void_p),
+        ("routing", C.c_uint32), ("num_identity_experts", C.c_uint32), ("selection_bias", C.c_void_p),
     ]
 
 
@@ -87,6 +91,11 @@ class LayerDesc(C.Structure):
         ("has_ple", C.c_uint32), ("ple_dim", C.c_uint32), ("ple_activation", C.c_uint32), ("is_non_causal", C.c_uint32),
         ("ple_gate", LinearDesc), ("ple_projection", LinearDesc), ("ple_norm", NormDesc),
         ("moe", MoeDesc),
+        # layer mechanisms of the f32-stream designs (all zero / NULL = none)
+        ("latent_rank", C.c_uint32), ("value_head_dim", C.c_uint32),
+        ("latent_down", LinearDesc), ("latent_norm", NormDesc), ("latent_up_keys", LinearDesc), ("latent_up_values", LinearDesc),
+        ("token_shift", C.c_void_p), ("depth_weights", C.c_void_p),
+        ("num_depth_weights", C.c_uint32), ("mlp_plain", C.c_uint32), ("no_mlp", C.c_uint32), ("reserved4", C.c_uint32),
     ]
 
 
@@ -106,6 +115,7 @@ class ModelDesc(C.Structure):
         ("ple_dim", C.c_uint32), ("ple_vocab_size", C.c_uint32), ("ple_embed_scale", C.c_float),
         ("ple_model_projection_scale", C.c_float), ("ple_input_scale", C.c_float), ("reserved", C.c_uint32),
         ("ple_token_embedding", LinearDesc), ("ple_model_projection", LinearDesc), ("ple_projection_norm", NormDesc),
+        ("f32_stream", C.c_uint32), ("reserved5", C.c_uint32),
     ]
 
 
@@ -166,10 +176,12 @@ class NormWeights:
     scale_offset: float = 0.0
     scales: Optional[np.ndarray] = None  # f32 [dim]
     biases: Optional[np.ndarray] = None
+    kind: int = NORM_STATISTICS          # NORM_DYNAMIC_TANH: tanh(alpha * x) * scales + biases (f32-stream designs)
+    alpha: float = 0.0
 
     def desc(self) -> NormDesc:
-        return NormDesc(int(self.present), int(self.full_layer), int(self.subtract_mean), 0, self.epsilon,
-                        self.scale_offset, _ptr(self.scales), _ptr(self.biases))
+        return NormDesc(int(self.present), int(self.full_layer), int(self.subtract_mean), int(self.kind), self.epsilon,
+                        self.scale_offset, _ptr(self.scales), _ptr(self.biases), float(self.alpha), 0)
 
 
 ABSENT_NORM = NormWeights(present=False)
@@ -205,26 +217,32 @@ class MoeWeights:
     num_active_experts: int
     expert_hidden_dim: int
     router_weights: np.ndarray   # [E, model_dim]
-    router_biases: np.ndarray    # [E]
-    w13: np.ndarray              # [E, 2 * d_ff, model_dim]
-    w2: np.ndarray               # [E, model_dim, d_ff]
-    up_biases: np.ndarray        # [E, 2 * d_ff]
-    down_biases: np.ndarray      # [E, model_dim]
+    router_biases: Optional[np.ndarray]    # [E]
+    w13: Optional[np.ndarray]              # [E, 2 * d_ff, model_dim]
+    w2: Optional[np.ndarray]               # [E, model_dim, d_ff]
+    up_biases: Optional[np.ndarray]        # [E, 2 * d_ff]
+    down_biases: Optional[np.ndarray]      # [E, model_dim]
     router_renorm: bool = True   # SoftmaxRouting
     gating_sel: int = 2          # 2 SwiGLU (SiLU), 3 GEGLU (GELUApprox)
     silu_alpha: float = 1.0
     gate_clip: tuple = (float("-inf"), float("inf"))
     up_clip: tuple = (float("-inf"), float("inf"))
+    # score routing (f32-stream designs): softmax over all router outputs, choice by score + selection_bias, weights = chosen scores / their sum; the last
+    # num_identity_experts router outputs return their input and have no tensors; no biases anywhere; router_weights is [E + identity, model_dim]
+    routing: int = MOE_ROUTE_TOPK_LOGITS
+    num_identity_experts: int = 0
+    selection_bias: Optional[np.ndarray] = None  # f32 [E + identity]
 
     def desc(self) -> MoeDesc:
         return MoeDesc(self.num_routed_experts, self.num_active_experts, self.expert_hidden_dim, int(self.router_renorm), self.gating_sel, self.silu_alpha,
                        self.gate_clip[0], self.gate_clip[1], self.up_clip[0], self.up_clip[1], _ptr(self.router_weights), _ptr(self.router_biases), _ptr(self.w13),
-                       _ptr(self.w2), _ptr(self.up_biases), _ptr(self.down_biases))
+                       _ptr(self.w2), _ptr(self.up_biases), _ptr(self.down_biases), int(self.routing), int(self.num_identity_experts), _ptr(self.selection_bias))
 
     def nbytes_active(self) -> int:
         """bytes one decoded token streams: the router + the k active experts' matrices and biases"""
-        per_expert = (self.w13.nbytes + self.w2.nbytes + self.up_biases.nbytes + self.down_biases.nbytes) // self.num_routed_experts
-        return self.router_weights.nbytes + self.router_biases.nbytes + self.num_active_experts * per_expert
+        nb = lambda a: 0 if a is None else a.nbytes
+        per_expert = (nb(self.w13) + nb(self.w2) + nb(self.up_biases) + nb(self.down_biases)) // max(self.num_routed_experts, 1)
+        return self.router_weights.nbytes + nb(self.router_biases) + self.num_active_experts * per_expert
 
 
 @dataclass
@@ -274,6 +292,18 @@ class LayerWeights:
     ple: Optional["PleLayerWeights"] = None      # ple_config: PerLayerEmbeddingProjection at the end of the layer
     is_non_causal: bool = False                  # AttentionConfig::is_causal == false (the block attention of a DFlash draft layer)
     moe: Optional["MoeWeights"] = None           # mlp_config = MixtureOfExpertsConfig: replaces the dense MLP (up / down projection are then None)
+    # f32-stream designs: latent attention (mixer_kind MIXER_LATENT_ATTENTION reuses num_heads / head_dim / attention_scale / sliding_window_size / sinks /
+    # kv_source_layer_index / qkv_projection (queries) / out_projection), token shift, depth mix, plain or absent MLP
+    latent_rank: int = 0
+    value_head_dim: int = 0
+    latent_down: Optional[LinearWeights] = None
+    latent_norm: NormWeights = field(default_factory=lambda: ABSENT_NORM)
+    latent_up_keys: Optional[LinearWeights] = None
+    latent_up_values: Optional[LinearWeights] = None
+    token_shift: Optional[np.ndarray] = None     # f32 [model_dim]
+    depth_weights: Optional[np.ndarray] = None   # f32 [layer + 2]
+    mlp_plain: bool = False
+    no_mlp: bool = False
 
     def desc(self) -> LayerDesc:
         empty = LinearDesc()
@@ -299,11 +329,13 @@ class LayerWeights:
             ld(self.ple.gate if self.ple else None), ld(self.ple.projection if self.ple else None),
             (self.ple.norm if self.ple else ABSENT_NORM).desc(),
             self.moe.desc() if self.moe is not None else MoeDesc(),
+            int(self.latent_rank), int(self.value_head_dim), ld(self.latent_down), self.latent_norm.desc(), ld(self.latent_up_keys), ld(self.latent_up_values),
+            _ptr(self.token_shift), _ptr(self.depth_weights), 0 if self.depth_weights is None else int(self.depth_weights.size), int(self.mlp_plain), int(self.no_mlp), 0,
         )
 
     def linears(self):
         names = ("qkv_projection", "gate_projection", "out_projection", "dn_in_proj", "dn_out_proj", "up_projection",
-                 "down_projection")
+                 "down_projection", "latent_down", "latent_up_keys", "latent_up_values")
         out = [(n, getattr(self, n)) for n in names if getattr(self, n) is not None]
         if self.ple is not None:
             out += [("ple.gate", self.ple.gate), ("ple.projection", self.ple.projection)]
@@ -462,6 +494,8 @@ class ModelBundle:
     ropes: Optional[List[RopeConfig]] = None     # distinct per-layer RoPE configurations (LayerWeights.rope_index); None: `rope` for all
     embedding_norm: NormWeights = field(default_factory=lambda: ABSENT_NORM)
     ple: Optional[PleModelWeights] = None
+    f32_stream: bool = False                     # an f32-stream design (include/uzu_model_desc.h): its own forward encoder, f32 logits, batched steps
+    architecture: Optional[str] = None           # config.json `architecture` of a design that is not in the reference's config schema
     _keep: list = field(default_factory=list, repr=False)
 
     def desc(self) -> ModelDesc:
@@ -484,7 +518,7 @@ class ModelBundle:
                          p.ple_dim if p else 0, p.ple_vocab_size if p else 0, p.ple_embed_scale if p else 0.0,
                          p.model_projection_scale if p else 0.0, p.input_scale if p else 0.0, 0,
                          p.token_embedding.desc() if p else e, p.model_projection.desc() if p else e,
-                         (p.projection_norm if p else ABSENT_NORM).desc())
+                         (p.projection_norm if p else ABSENT_NORM).desc(), int(self.f32_stream), 0)
 
     # ---- algorithmic bytes per decoded token (SURVEY.md §8d formula) ----
     def weight_stream_bytes(self) -> int:
@@ -506,6 +540,9 @@ class ModelBundle:
             if l.mixer_kind == MIXER_ATTENTION:
                 rows = min(context, l.sliding_window_size) if l.sliding_window_size else context
                 total += 2 * rows * l.num_groups * l.head_dim * 2             # K and V rows, bf16 (a sharing layer reads its source's)
+            elif l.mixer_kind == MIXER_LATENT_ATTENTION:
+                rows = min(context, l.sliding_window_size) if l.sliding_window_size else context
+                total += rows * l.latent_rank * 2                             # one latent row per visible token, bf16, shared by all heads
             else:
                 total += 2 * l.dn_num_heads * l.dn_value_head_dim * l.dn_head_dim * 4  # f32 state read + write
                 conv_dim = 2 * l.dn_num_groups * l.dn_head_dim + l.dn_num_heads * l.dn_value_head_dim
@@ -530,6 +567,10 @@ class ModelBundle:
         for l in self.layers:
             if l.mixer_kind == MIXER_ATTENTION:
                 flops += 4.0 * pairs * l.num_heads * l.head_dim
+            elif l.mixer_kind == MIXER_LATENT_ATTENTION:  # scores and weighted sum in latent space, over the window
+                w = l.sliding_window_size
+                vis = pairs if not w else min(pairs, tokens * float(w))
+                flops += 4.0 * vis * l.num_heads * l.latent_rank
             else:  # delta rule: ~6 flops per state element per token (decay, S k, rank-1 update, S q)
                 flops += 6.0 * tokens * l.dn_num_heads * l.dn_value_head_dim * l.dn_head_dim
         return flops

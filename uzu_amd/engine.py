@@ -16,7 +16,7 @@ from ._ffi import call
 from .backend import Context
 from .desc import ModelBundle
 
-MODEL_DEFAULT, MODEL_NO_GRAPH, MODEL_NO_FUSION, MODEL_DEBUG_TAPS = 0, 1, 2, 4
+MODEL_DEFAULT, MODEL_NO_GRAPH, MODEL_NO_FUSION, MODEL_DEBUG_TAPS, MODEL_FULL_F32 = 0, 1, 2, 4, 8
 
 
 def check_desc_abi():
@@ -80,6 +80,7 @@ class HipModel:
         self.vocab_size = bundle.vocab_size
         self.model_dim = bundle.model_dim
         self.num_layers = len(bundle.layers)
+        self.f32_stream = bool(getattr(bundle, "f32_stream", False))
         self.tp_group = tp_group
         check_desc_abi()
         desc = bundle.desc()
@@ -123,6 +124,44 @@ class HipModel:
         call("uzu_hip_model_prefill_batch", self._h, handles, C.c_uint32(len(states)), C.c_void_p(tokens.ctypes.data), C.c_uint32(tokens.shape[1]),
              C.c_void_p(first.ctypes.data))
         return first
+
+    def step_batch(self, states, tokens, want=None, sample: bool = False):
+        """One batched step of an f32-stream design (uzu_hip_model_step_batch): `tokens[i]` = the next tokens of `states[i]` (any lengths >= 1; prefill and
+        batched decode alike).  `want[i]` = positions inside tokens[i] whose logits are wanted.  Returns (logits f32 [sum of wants, vocab] in the order of the
+        sequences and of their `want`, sampled tokens [len(states)] or None)."""
+        counts = np.asarray([len(t) for t in tokens], dtype=np.uint32)
+        flat = np.ascontiguousarray(np.concatenate([np.asarray(t, dtype=np.uint32) for t in tokens]))
+        offs = np.concatenate([[0], np.cumsum(counts)])
+        rows = [int(offs[i]) + int(p) for i, w in enumerate(want or []) for p in w]
+        order = sorted(set(rows))
+        want_rows = np.asarray(order, dtype=np.uint32)
+        logits = np.empty((len(order), self.vocab_size), dtype=np.float32)
+        sampled = np.zeros(len(states), dtype=np.uint32) if sample else None
+        arr = (C.c_void_p * len(states))(*[s._h for s in states])
+        call("uzu_hip_model_step_batch", self._h, arr, C.c_uint32(len(states)), flat.ctypes.data_as(C.c_void_p), counts.ctypes.data_as(C.c_void_p),
+             want_rows.ctypes.data_as(C.c_void_p) if len(order) else None, C.c_uint32(len(order)), logits.ctypes.data_as(C.c_void_p) if len(order) else None,
+             sampled.ctypes.data_as(C.c_void_p) if sample else None)
+        if rows != order:
+            index = {r: i for i, r in enumerate(order)}
+            logits = logits[[index[r] for r in rows]]
+        return logits, sampled
+
+    def read_logits_f32(self, row: Optional[int] = None) -> np.ndarray:
+        """f32 logits of one row of the last read-out of an f32-stream design (default: the last row = the sampled one)"""
+        fn = _ffi.lib().uzu_hip_model_logit_rows
+        fn.restype, fn.argtypes = C.c_uint32, [C.c_void_p]
+        n = fn(self._h)
+        out = np.empty(self.vocab_size, dtype=np.float32)
+        call("uzu_hip_model_read_logits_f32", self._h, C.c_uint32(n - 1 if row is None else row), out.ctypes.data_as(C.c_void_p))
+        return out
+
+    def read_layer_output_f32(self, layer: int) -> np.ndarray:
+        """MODEL_DEBUG_TAPS on an f32-stream design: f32 [rows, model_dim], what `layer` handed on in the last pass"""
+        rows = C.c_uint32()
+        call("uzu_hip_model_read_layer_output_f32", self._h, C.c_uint32(layer), None, C.byref(rows))
+        out = np.empty((rows.value, self.model_dim), dtype=np.float32)
+        call("uzu_hip_model_read_layer_output_f32", self._h, C.c_uint32(layer), out.ctypes.data_as(C.c_void_p), C.byref(rows))
+        return out
 
     @property
     def context_length(self) -> int:

@@ -115,6 +115,25 @@ uzu_status uzu_hip_model_read_logits_f32(uzu_hip_model* m, uint32_t row, float* 
 uint32_t uzu_hip_model_logit_rows(const uzu_hip_model* m);
 /* UZU_MODEL_DEBUG_TAPS on an f32-stream design: f32 [rows, model_dim], what `layer` handed on in the last pass (`out` NULL: rows only) */
 uzu_status uzu_hip_model_read_layer_output_f32(uzu_hip_model* m, uint32_t layer, float* out, uint32_t* rows);
+/* The kernels of the f32-stream designs one by one, for ONE sequence, host arrays in and out (csrc/capi_stream32.hip): what the parity tests hold to an
+ * independent statement of each mechanism.  `bf16_products`: round the activation operand of a product to bf16 (the serving precision); 0: true f32.
+ *   linear: y[r][b*n + j] = act(sum_k x[r][b*k' + k] w[b][j][k] + bias[j]) + residual; batch > 1 = the per-head products; form 0 dispatch, 1 matrix cores, 2 not.
+ *   dyn_tanh: tanh(alpha x) scales + biases, then (shift != NULL) the token shift from prev_inout (state row in, state row out) at position `start`.
+ *   latent_norm_append: RMS-normalised latents of positions start.. into cache_inout [(start + rows)][rank].
+ *   latent_attention: latent-space attention core over cache [(start + rows)][rank]; form 0 dispatch, 1 simple, 2 tiled.
+ *   moe: score routing (softmax over routed + identity outputs, choice by score + selection_bias) + SiLU-gated experts + identity experts + residual. */
+uzu_status uzu_hip_s32_linear(uzu_hip_context* ctx, const float* x, const uint16_t* w, const uint16_t* bias, const float* residual, float* y, uint32_t rows, uint32_t n, uint32_t k,
+                              uint32_t batch, uint32_t act, uint32_t bf16_products, uint32_t form);
+uzu_status uzu_hip_s32_dyn_tanh(uzu_hip_context* ctx, const float* x, const float* scales, const float* biases, float alpha, const float* shift, float* prev_inout, uint32_t start,
+                                float* out, uint32_t rows, uint32_t d);
+uzu_status uzu_hip_s32_depth_mix(uzu_hip_context* ctx, const float* slots, const float* w, uint32_t count, float* out, uint32_t rows, uint32_t d);
+uzu_status uzu_hip_s32_latent_norm_append(uzu_hip_context* ctx, const float* x, const float* scales, float eps, float* cache_inout, uint32_t cache_bf16, uint32_t start, uint32_t rows,
+                                          uint32_t rank);
+uzu_status uzu_hip_s32_latent_attention(uzu_hip_context* ctx, const float* qlat, const float* cache, const float* sinks, float* out, uint32_t rows, uint32_t start, uint32_t heads,
+                                        uint32_t rank, uint32_t window, float scale, uint32_t cache_bf16, uint32_t form);
+uzu_status uzu_hip_s32_moe(uzu_hip_context* ctx, const float* x, const uint16_t* router, const float* selection_bias, const uint16_t* w13, const uint16_t* w2, const float* residual,
+                           float* y, int32_t* ids_out, float* weights_out, uint32_t rows, uint32_t d, uint32_t ff, uint32_t routed, uint32_t identity, uint32_t top,
+                           uint32_t bf16_products);
 /* LanguageModelState reset: context length 0, DeltaNet conv / SSM state zeroed. */
 uzu_status uzu_hip_model_reset(uzu_hip_model* m);
 uint32_t uzu_hip_model_context_length(const uzu_hip_model* m);

@@ -1,0 +1,204 @@
+"""Lazolix through the engine (HipModel: states, batched steps, prefill / decode, sampling) against the float64 oracle on small models of the tests' own making:
+sizes that are not powers of two, head widths that differ between queries and values, layers with and without window / MLP / shared latents, one and no
+identity expert, one and several winners."""
+import numpy as np
+import pytest
+
+import lazolix_oracle as O
+from uzu_amd import loader
+from uzu_amd.engine import MODEL_BATCH, MODEL_DEBUG_TAPS, MODEL_FULL_F32, HipModel
+
+pytestmark = pytest.mark.gpu
+
+TOL = {True: 4e-5, False: 6e-2}  # full f32 / bf16 products: rms logit error relative to the rms of the logits
+
+
+def cfg_a():
+    return O.config(vocab=61, width=40, layers=[
+        O.layer(3, 8, 16, 24, window=5, mlp=O.dense(72)),
+        O.layer(2, 16, 8, 24, window=None, kv_from=0, scale=0.2, mlp=O.moe(3, 2, 16, identity=1)),
+        O.layer(1, 24, 8, 16, window=1, mlp=None),
+        O.layer(5, 8, 8, 16, window=3, kv_from=2, mlp=O.moe(2, 1, 24, identity=0)),
+    ])
+
+
+def cfg_b():  # matrix-core friendly sizes: rank and widths in multiples of 8, a window that spans several key blocks
+    return O.config(vocab=97, width=64, layers=[
+        O.layer(4, 16, 16, 64, window=40, mlp=O.moe(4, 2, 32, identity=2)),
+        O.layer(8, 8, 16, 64, window=None, kv_from=0, mlp=O.dense(96)),
+        O.layer(2, 32, 8, 128, window=70, mlp=O.moe(1, 1, 16, identity=1)),
+    ], eps=1e-5)
+
+
+@pytest.fixture(scope="module")
+def models(hip_ctx, tmp_path_factory):
+    out = {}
+    for name, cfg, seed in (("a", cfg_a(), 11), ("b", cfg_b(), 12)):
+        W = O.weights(cfg, seed)
+        path = str(tmp_path_factory.mktemp("lazolix") / name)
+        O.write_model_dir(path, cfg, W)
+        bundle = loader.load_model_dir(path, max_context_length=512)
+        W64 = {k: v.astype(np.float64) for k, v in W.items()}
+        out[name] = (cfg, W64, {full: HipModel(hip_ctx, bundle, MODEL_BATCH(6) | MODEL_DEBUG_TAPS | (MODEL_FULL_F32 if full else 0)) for full in (True, False)})
+    yield out
+    for _, _, ms in out.values():
+        for m in ms.values():
+            m.close()
+
+
+def prompt(cfg, n, seed):
+    return list(np.random.default_rng(seed).integers(0, cfg["vocab"], size=n))
+
+
+@pytest.mark.parametrize("name", ["a", "b"])
+@pytest.mark.parametrize("full", [True, False])
+def test_whole_prompt_every_position_and_every_layer(models, name, full):
+    cfg, W, ms = models[name]
+    m = ms[full]
+    toks = prompt(cfg, 150, 1)
+    layers = []
+    want = O.forward(cfg, W, toks, layers)
+    st = m.new_state()
+    got, _ = m.step_batch([st], [toks], [list(range(len(toks)))])
+    for l, ref in enumerate(layers):  # the residual stream behind every layer: names the first layer that differs
+        err = np.abs(m.read_layer_output_f32(l) - ref).max() / np.abs(ref).max()
+        assert err < (2e-5 if full else 5e-2), (l, err)
+    assert O.logit_error(got, want).max() < TOL[full]
+    st.close()
+
+
+@pytest.mark.parametrize("name", ["a", "b"])
+@pytest.mark.parametrize("full", [True, False])
+def test_prefill_then_token_by_token_and_portions_down_to_two_tokens(models, name, full):
+    cfg, W, ms = models[name]
+    m = ms[full]
+    toks = prompt(cfg, 120, 2)
+    want = O.forward(cfg, W, toks)
+    for cuts in ([100] + [1] * 20, [1] * 30 + [90], [2, 3, 2, 50, 7, 2, 54], [33, 31, 17, 39]):
+        assert sum(cuts) == len(toks)
+        st, rows, at = m.new_state(), [], 0
+        for n in cuts:
+            lg, _ = m.step_batch([st], [toks[at:at + n]], [list(range(n))])
+            rows.append(lg)
+            at += n
+        assert st.context_length == len(toks)
+        assert O.logit_error(np.concatenate(rows), want).max() < TOL[full], cuts
+        st.close()
+
+
+@pytest.mark.parametrize("name", ["a", "b"])
+def test_unequal_batch_equals_each_request_alone_and_reused_states(models, name):
+    cfg, W, ms = models[name]
+    m = ms[True]
+    reqs = [prompt(cfg, n, 10 + n) for n in (1, 37, 90, 5, 64)]
+    alone = []
+    for r in reqs:
+        st = m.new_state()
+        first, _ = m.step_batch([st], [r[:-3]] if len(r) > 3 else [r], [[len(r) - 4] if len(r) > 3 else [0]])
+        tail = [m.step_batch([st], [[t]], [[0]])[0] for t in (r[-3:] if len(r) > 3 else [])]
+        alone.append(np.concatenate([first] + tail))
+        st.close()
+    pool = [m.new_state() for _ in reqs]
+    for round_ in range(2):  # the second round reuses the states the first one gave back (reset), in another order
+        states = pool if round_ == 0 else pool[::-1]
+        heads = [r[:-3] if len(r) > 3 else r for r in reqs]
+        lg, _ = m.step_batch(states, heads, [[len(h) - 1] for h in heads])
+        got = [[lg[i]] for i in range(len(reqs))]
+        for step in range(3):  # decoded together; the one-token request has left the batch
+            live = [i for i, r in enumerate(reqs) if len(r) > 3]
+            lg, _ = m.step_batch([states[i] for i in live], [[reqs[i][len(reqs[i]) - 3 + step]] for i in live], [[0]] * len(live))
+            for row, i in zip(lg, live):
+                got[i].append(row)
+        for i in range(len(reqs)):
+            assert np.abs(np.stack(got[i]) - alone[i]).max() < 2e-4 * np.abs(alone[i]).max(), (round_, i)
+            assert O.logit_error(np.stack(got[i])[-1:], O.forward(cfg, W, reqs[i])[-1:]).max() < TOL[True]
+        for st in states:
+            st.reset()
+    for st in pool:
+        st.close()
+
+
+def test_more_requests_than_a_pass_carries_and_prompts_longer_than_a_pass(hip_ctx, tmp_path):
+    cfg = O.config(vocab=31, width=16, layers=[O.layer(2, 8, 8, 8, window=6, mlp=O.dense(24)), O.layer(2, 8, 8, 8, window=None, kv_from=0, mlp=None)])
+    W = O.weights(cfg, 21)
+    O.write_model_dir(str(tmp_path / "m"), cfg, W)
+    W64 = {k: v.astype(np.float64) for k, v in W.items()}
+    m = HipModel(hip_ctx, loader.load_model_dir(str(tmp_path / "m"), max_context_length=3000), MODEL_BATCH(2) | MODEL_FULL_F32)
+    reqs = [prompt(cfg, n, n) for n in (9, 2100, 4, 30, 2)]  # 2100 > one pass of 2048 rows; five requests > two per pass
+    states = [m.new_state() for _ in reqs]
+    lg, sampled = m.step_batch(states, reqs, [[len(r) - 1] for r in reqs], sample=True)
+    for i, r in enumerate(reqs):
+        want = O.forward(cfg, W64, r)[-1:] if len(r) < 200 else None
+        if want is not None:
+            assert O.logit_error(lg[i:i + 1], want).max() < TOL[True] and int(sampled[i]) == int(np.argmax(want))
+        assert states[i].context_length == len(r)
+    # the long prompt: against the same prompt through two explicit portions
+    st = m.new_state()
+    m.step_batch([st], [reqs[1][:1500]], [[]])
+    two, _ = m.step_batch([st], [reqs[1][1500:]], [[599]])
+    assert np.abs(two[0] - lg[1]).max() < 2e-4 * np.abs(two).max()
+    m.close()
+
+
+@pytest.mark.parametrize("full", [True, False])
+def test_long_decoding_across_windows(models, full):
+    cfg, W, ms = models["b"]
+    m = ms[full]
+    toks = prompt(cfg, 230, 5)
+    want = O.forward(cfg, W, toks)
+    st = m.new_state()
+    m.step_batch([st], [toks[:10]], [[]])
+    rows = [m.step_batch([st], [[t]], [[0]])[0][0] for t in toks[10:]]  # 220 decoded tokens: every window (40, 70) slides over decoded tokens only
+    assert O.logit_error(np.stack(rows), want[10:]).max() < TOL[full]
+    st.close()
+
+
+@pytest.mark.parametrize("name", ["a", "b"])
+def test_greedy_generation_through_prefill_and_decode(models, name):
+    """The engine's own entry points: HipModel.prefill + chained decode (the sampled token is fed back on the device), then the stochastic sampler's plumbing."""
+    cfg, W, ms = models[name]
+    m = ms[True]
+    p = prompt(cfg, 25, 7)
+    m.reset()
+    m.set_sampling(None)
+    first = m.prefill(np.asarray(p, dtype=np.uint32))
+    rest, _ = m.decode(9)
+    got = [int(first)] + [int(t) for t in rest]
+    want, margin_ok = [], True
+    toks = list(p)
+    for _ in range(10):
+        row = O.forward(cfg, W, toks)[-1]
+        top2 = np.sort(row)[-2:]
+        margin_ok = margin_ok and (top2[1] - top2[0]) > 1e-3 * np.abs(row).max()
+        want.append(int(np.argmax(row)))
+        toks.append(want[-1])
+    assert margin_ok, "the oracle's own greedy stream has a near tie: pick another seed"
+    assert got == want and m.context_length == len(p) + 9
+    assert np.argmax(m.read_logits_f32()) == want[-1]
+    # temperature -> 0 of the stochastic sampler is greedy; a fixed seed repeats
+    m.reset()
+    m.set_sampling(seed=3, temperature=1e-4)
+    s1 = [int(m.prefill(np.asarray(p, dtype=np.uint32)))] + [int(t) for t in m.decode(4)[0]]
+    assert s1 == want[:5]
+    m.reset()
+    m.set_sampling(seed=5, temperature=1.5, top_k=7)
+    a = [int(m.prefill(np.asarray(p, dtype=np.uint32)))] + [int(t) for t in m.decode(6)[0]]
+    m.reset()
+    b = [int(m.prefill(np.asarray(p, dtype=np.uint32)))] + [int(t) for t in m.decode(6)[0]]
+    assert a == b
+    m.set_sampling(None)
+    m.reset()
+
+
+def test_refusals(models, hip_ctx):
+    cfg, W, ms = models["a"]
+    m = ms[True]
+    st = m.new_state()
+    from uzu_amd._ffi import UzuHipError
+    with pytest.raises(UzuHipError):
+        m.step_batch([st], [[cfg["vocab"]]], [[0]])          # a token id outside the vocabulary
+    with pytest.raises(UzuHipError):
+        m.step_batch([st, st], [[1], [2]], [[0], [0]])       # one state twice in a batch
+    with pytest.raises(UzuHipError):
+        m.step_batch([st], [[1] * 600], [[]])                # beyond max_context_length
+    st.close()

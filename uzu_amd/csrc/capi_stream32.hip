@@ -1,0 +1,229 @@
+// capi_stream32.hip -- the kernels of the f32-stream designs behind plain C entries (include/uzu_hip_engine.h): host arrays in, host arrays out, ONE sequence.
+// They exist so that every mechanism can be held to an independent statement of its equations on its own (tests/test_gpu_lazolix_kernels.py) and so that two
+// forms of one kernel can be compared on the same inputs; the engine calls the kernels directly (engine_stream32.hip).
+#include <vector>
+
+#include "device_utils.h"
+#include "kernels_stream32.h"
+
+using namespace uzu;
+
+namespace {
+
+struct Scratch { // device allocations of one call
+    std::vector<void*> ptrs;
+    ~Scratch() {
+        for (void* p : ptrs) (void)hipFree(p);
+    }
+    template <class T> uzu_status up(const T* host, size_t count, T** out) {
+        *out = nullptr;
+        if (!count) return UZU_OK;
+        void* p = nullptr;
+        UZU_HIP_TRY(hipMalloc(&p, count * sizeof(T) + 256));
+        ptrs.push_back(p);
+        if (host) UZU_HIP_TRY(hipMemcpy(p, host, count * sizeof(T), hipMemcpyHostToDevice));
+        else UZU_HIP_TRY(hipMemset(p, 0xFF, count * sizeof(T))); // an output: what the kernel does not write reads as NaN
+        *out = (T*)p;
+        return UZU_OK;
+    }
+};
+
+uzu_status one_sequence(Scratch& S, uint32_t rows, uint32_t start, k::SeqSpan** spans, uint32_t** row_seq) {
+    const k::SeqSpan sp{0, rows, start};
+    std::vector<uint32_t> zeros(rows, 0u);
+    UZU_PROPAGATE(S.up(&sp, 1, spans));
+    return S.up(zeros.data(), rows, row_seq);
+}
+
+uzu_status finish(uzu_hip_context* ctx) {
+    UZU_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return UZU_OK;
+}
+
+} // namespace
+
+extern "C" {
+
+uzu_status uzu_hip_s32_linear(uzu_hip_context* ctx, const float* x, const uint16_t* w, const uint16_t* bias, const float* residual, float* y, uint32_t rows, uint32_t n, uint32_t kk,
+                              uint32_t batch, uint32_t act, uint32_t bf16_products, uint32_t form) {
+    UZU_REQUIRE(ctx && x && w && y && batch, "s32_linear: null argument");
+    (void)hipSetDevice(ctx->device);
+    Scratch S;
+    k::LinearF32Params p{};
+    float *dx, *dy, *dr = nullptr;
+    uint16_t *dw, *db = nullptr;
+    // batch > 1: x [rows][batch * k], w [batch][n][k], y [rows][batch * n] (the per-head products of the attention)
+    UZU_PROPAGATE(S.up(x, (size_t)rows * kk * batch, &dx));
+    UZU_PROPAGATE(S.up(w, (size_t)n * kk * batch, &dw));
+    if (bias) UZU_PROPAGATE(S.up(bias, n, &db));
+    if (residual) UZU_PROPAGATE(S.up(residual, (size_t)rows * n, &dr));
+    UZU_PROPAGATE(S.up((const float*)nullptr, (size_t)rows * n * batch, &dy));
+    p.x = dx, p.w = dw, p.bias = db, p.residual = dr, p.y = dy, p.rows = rows, p.n = n, p.k = kk, p.ldx = kk * batch, p.ldy = n * batch, p.ldr = n, p.batch = batch;
+    p.x_batch = kk, p.w_batch = (size_t)n * kk, p.y_batch = n, p.act = act, p.bf16_products = bf16_products;
+    if (form == 1) { // the matrix-core form or nothing
+        UZU_UNSUPPORTED(!k::linear_mfma_supported(p), "s32_linear: the matrix-core form does not take this shape");
+        UZU_PROPAGATE(k::linear_mfma(ctx->stream, p));
+    } else if (form == 2) { // without the matrix cores
+        k::LinearF32Params q = p;
+        q.bf16_products = 0; // (the dispatcher only offers the matrix cores to bf16 products)
+        if (bf16_products) { // round the operand here, then true f32 products: the same numbers as bf16 products
+            std::vector<float> xr((size_t)rows * kk * batch);
+            for (size_t i = 0; i < xr.size(); ++i) xr[i] = round_bf16(x[i]);
+            UZU_HIP_TRY(hipMemcpy(dx, xr.data(), xr.size() * 4, hipMemcpyHostToDevice));
+        }
+        UZU_PROPAGATE(k::linear_f32(ctx->stream, q));
+    } else {
+        UZU_PROPAGATE(k::linear_f32(ctx->stream, p));
+    }
+    UZU_PROPAGATE(finish(ctx));
+    UZU_HIP_TRY(hipMemcpy(y, dy, (size_t)rows * n * batch * 4, hipMemcpyDeviceToHost));
+    return UZU_OK;
+}
+
+// prev_inout [d]: the sequence's last normalised row before the call / after it (token shift only)
+uzu_status uzu_hip_s32_dyn_tanh(uzu_hip_context* ctx, const float* x, const float* scales, const float* biases, float alpha, const float* shift, float* prev_inout, uint32_t start,
+                                float* out, uint32_t rows, uint32_t d) {
+    UZU_REQUIRE(ctx && x && scales && out && (!shift || prev_inout), "s32_dyn_tanh: null argument");
+    (void)hipSetDevice(ctx->device);
+    Scratch S;
+    k::DynTanhParams p{};
+    float *dx, *ds, *db = nullptr, *dsh = nullptr, *dprev = nullptr, *dout;
+    float** dpp = nullptr;
+    UZU_PROPAGATE(S.up(x, (size_t)rows * d, &dx));
+    UZU_PROPAGATE(S.up(scales, d, &ds));
+    if (biases) UZU_PROPAGATE(S.up(biases, d, &db));
+    UZU_PROPAGATE(S.up((const float*)nullptr, (size_t)rows * d, &dout));
+    p.x = dx, p.out = dout, p.scales = ds, p.biases = db, p.alpha = alpha, p.rows = rows, p.d = d;
+    if (shift) {
+        k::SeqSpan* spans;
+        uint32_t* row_seq;
+        UZU_PROPAGATE(S.up(shift, d, &dsh));
+        UZU_PROPAGATE(S.up((const float*)prev_inout, d, &dprev));
+        UZU_PROPAGATE(S.up((float* const*)&dprev, 1, &dpp));
+        UZU_PROPAGATE(one_sequence(S, rows, start, &spans, &row_seq));
+        p.shift = dsh, p.prev = dpp, p.spans = spans, p.row_seq = row_seq;
+    }
+    UZU_PROPAGATE(k::dyn_tanh_norm(ctx->stream, p));
+    UZU_PROPAGATE(finish(ctx));
+    UZU_HIP_TRY(hipMemcpy(out, dout, (size_t)rows * d * 4, hipMemcpyDeviceToHost));
+    if (shift) UZU_HIP_TRY(hipMemcpy(prev_inout, dprev, (size_t)d * 4, hipMemcpyDeviceToHost));
+    return UZU_OK;
+}
+
+uzu_status uzu_hip_s32_depth_mix(uzu_hip_context* ctx, const float* slots, const float* w, uint32_t count, float* out, uint32_t rows, uint32_t d) {
+    UZU_REQUIRE(ctx && slots && w && out, "s32_depth_mix: null argument");
+    (void)hipSetDevice(ctx->device);
+    Scratch S;
+    float *ds, *dw, *dout;
+    UZU_PROPAGATE(S.up(slots, (size_t)count * rows * d, &ds));
+    UZU_PROPAGATE(S.up(w, count, &dw));
+    UZU_PROPAGATE(S.up((const float*)nullptr, (size_t)rows * d, &dout));
+    UZU_PROPAGATE(k::depth_mix(ctx->stream, ds, (size_t)rows * d, dw, count, dout, rows, d));
+    UZU_PROPAGATE(finish(ctx));
+    UZU_HIP_TRY(hipMemcpy(out, dout, (size_t)rows * d * 4, hipMemcpyDeviceToHost));
+    return UZU_OK;
+}
+
+// x [rows][rank] raw latents of positions start ..; cache_out [(start + rows)][rank] f32: rows below `start` come back as given in cache_inout
+uzu_status uzu_hip_s32_latent_norm_append(uzu_hip_context* ctx, const float* x, const float* scales, float eps, float* cache_inout, uint32_t cache_bf16, uint32_t start, uint32_t rows,
+                                          uint32_t rank) {
+    UZU_REQUIRE(ctx && x && scales && cache_inout, "s32_latent_norm_append: null argument");
+    (void)hipSetDevice(ctx->device);
+    Scratch S;
+    const size_t total = (size_t)(start + rows) * rank;
+    float *dx, *ds, *dc32 = nullptr;
+    uint16_t* dc16 = nullptr;
+    void** dcp;
+    k::SeqSpan* spans;
+    uint32_t* row_seq;
+    UZU_PROPAGATE(S.up(x, (size_t)rows * rank, &dx));
+    UZU_PROPAGATE(S.up(scales, rank, &ds));
+    std::vector<uint16_t> bits(total);
+    if (cache_bf16) {
+        for (size_t i = 0; i < total; ++i) bits[i] = f32_to_bf16(cache_inout[i]);
+        UZU_PROPAGATE(S.up(bits.data(), total, &dc16));
+    } else {
+        UZU_PROPAGATE(S.up((const float*)cache_inout, total, &dc32));
+    }
+    void* cache = cache_bf16 ? (void*)dc16 : (void*)dc32;
+    UZU_PROPAGATE(S.up((void* const*)&cache, 1, &dcp));
+    UZU_PROPAGATE(one_sequence(S, rows, start, &spans, &row_seq));
+    UZU_PROPAGATE(k::latent_norm_append(ctx->stream, dx, ds, eps, dcp, cache_bf16, spans, row_seq, rows, rank));
+    UZU_PROPAGATE(finish(ctx));
+    if (cache_bf16) {
+        UZU_HIP_TRY(hipMemcpy(bits.data(), dc16, total * 2, hipMemcpyDeviceToHost));
+        for (size_t i = 0; i < total; ++i) cache_inout[i] = bf16_to_f32(bits[i]);
+    } else {
+        UZU_HIP_TRY(hipMemcpy(cache_inout, dc32, total * 4, hipMemcpyDeviceToHost));
+    }
+    return UZU_OK;
+}
+
+// qlat / out [rows][heads * rank] for positions start .. start + rows - 1; cache f32 [(start + rows)][rank] (rounded to bf16 here when cache_bf16).
+// form 0: the engine's choice for the shape; 1: the simple form (a wave per row and head); 2: the tiled form
+uzu_status uzu_hip_s32_latent_attention(uzu_hip_context* ctx, const float* qlat, const float* cache, const float* sinks, float* out, uint32_t rows, uint32_t start, uint32_t heads,
+                                        uint32_t rank, uint32_t window, float scale, uint32_t cache_bf16, uint32_t form) {
+    UZU_REQUIRE(ctx && qlat && cache && out, "s32_latent_attention: null argument");
+    (void)hipSetDevice(ctx->device);
+    Scratch S;
+    const size_t total = (size_t)(start + rows) * rank;
+    float *dq, *dout, *dsink = nullptr, *dc32 = nullptr;
+    uint16_t* dc16 = nullptr;
+    void** dcp;
+    k::SeqSpan* spans;
+    uint32_t* row_seq;
+    UZU_PROPAGATE(S.up(qlat, (size_t)rows * heads * rank, &dq));
+    UZU_PROPAGATE(S.up((const float*)nullptr, (size_t)rows * heads * rank, &dout));
+    if (sinks) UZU_PROPAGATE(S.up(sinks, heads, &dsink));
+    if (cache_bf16) {
+        std::vector<uint16_t> bits(total);
+        for (size_t i = 0; i < total; ++i) bits[i] = f32_to_bf16(cache[i]);
+        UZU_PROPAGATE(S.up(bits.data(), total, &dc16));
+    } else {
+        UZU_PROPAGATE(S.up(cache, total, &dc32));
+    }
+    void* cp = cache_bf16 ? (void*)dc16 : (void*)dc32;
+    UZU_PROPAGATE(S.up((void* const*)&cp, 1, &dcp));
+    UZU_PROPAGATE(one_sequence(S, rows, start, &spans, &row_seq));
+    k::LatentAttentionParams p{};
+    p.qlat = dq, p.out = dout, p.caches = dcp, p.cache_bf16 = cache_bf16, p.sinks = dsink, p.spans = spans, p.row_seq = row_seq;
+    p.rows = rows, p.heads = heads, p.rank = rank, p.window = window, p.scale = scale, p.form = form, p.nseq = 1, p.tiles = (rows * heads + 127) / 128;
+    UZU_PROPAGATE(k::latent_attention(ctx->stream, p));
+    UZU_PROPAGATE(finish(ctx));
+    UZU_HIP_TRY(hipMemcpy(out, dout, (size_t)rows * heads * rank * 4, hipMemcpyDeviceToHost));
+    return UZU_OK;
+}
+
+// the whole score-routed block on rows x: ids / weights [rows][top] and y = residual + sum of the winners' outputs
+uzu_status uzu_hip_s32_moe(uzu_hip_context* ctx, const float* x, const uint16_t* router, const float* selection_bias, const uint16_t* w13, const uint16_t* w2, const float* residual,
+                           float* y, int32_t* ids_out, float* weights_out, uint32_t rows, uint32_t d, uint32_t ff, uint32_t routed, uint32_t identity, uint32_t top,
+                           uint32_t bf16_products) {
+    UZU_REQUIRE(ctx && x && router && y && (!routed || (w13 && w2)), "s32_moe: null argument");
+    (void)hipSetDevice(ctx->device);
+    Scratch S;
+    float *dx, *dsb = nullptr, *dres = nullptr, *dy, *dwt, *dh;
+    uint16_t *dr, *d13 = nullptr, *d2 = nullptr;
+    int32_t* dids;
+    UZU_PROPAGATE(S.up(x, (size_t)rows * d, &dx));
+    UZU_PROPAGATE(S.up(router, (size_t)(routed + identity) * d, &dr));
+    if (selection_bias) UZU_PROPAGATE(S.up(selection_bias, routed + identity, &dsb));
+    if (routed) {
+        UZU_PROPAGATE(S.up(w13, (size_t)routed * 2 * ff * d, &d13));
+        UZU_PROPAGATE(S.up(w2, (size_t)routed * d * ff, &d2));
+    }
+    if (residual) UZU_PROPAGATE(S.up(residual, (size_t)rows * d, &dres));
+    UZU_PROPAGATE(S.up((const float*)nullptr, (size_t)rows * d, &dy));
+    UZU_PROPAGATE(S.up((const float*)nullptr, (size_t)rows * top, &dwt));
+    UZU_PROPAGATE(S.up((const float*)nullptr, (size_t)rows * top * (ff ? ff : 1), &dh));
+    UZU_PROPAGATE(S.up((const int32_t*)nullptr, (size_t)rows * top, &dids));
+    UZU_PROPAGATE(k::moe_route_scores(ctx->stream, dx, dr, dsb, dids, dwt, rows, d, routed + identity, top));
+    UZU_PROPAGATE(k::moe_experts_gate_up(ctx->stream, dx, dids, d13, dh, rows, d, ff, routed, top, bf16_products));
+    UZU_PROPAGATE(k::moe_experts_down_combine(ctx->stream, dh, dx, dids, dwt, d2, dres, dy, rows, d, ff, routed, top, bf16_products));
+    UZU_PROPAGATE(finish(ctx));
+    UZU_HIP_TRY(hipMemcpy(y, dy, (size_t)rows * d * 4, hipMemcpyDeviceToHost));
+    if (ids_out) UZU_HIP_TRY(hipMemcpy(ids_out, dids, (size_t)rows * top * 4, hipMemcpyDeviceToHost));
+    if (weights_out) UZU_HIP_TRY(hipMemcpy(weights_out, dwt, (size_t)rows * top * 4, hipMemcpyDeviceToHost));
+    return UZU_OK;
+}
+
+} // extern "C"

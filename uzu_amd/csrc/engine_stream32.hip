@@ -165,6 +165,8 @@ uzu_status s32_pass(uzu_hip_model* m, const std::vector<PassSeq>& seqs, const ui
             ap.qlat = S.qlat, ap.out = S.ctx, ap.caches = caches, ap.cache_bf16 = bf, ap.sinks = X.sinks, ap.spans = S.d_spans, ap.row_seq = S.d_row_seq;
             ap.rows = rows, ap.heads = H, ap.rank = rank, ap.window = h.sliding_window_size;
             ap.scale = h.attention_scale != 0.0f ? h.attention_scale : 1.0f / sqrtf((float)hd);
+            ap.nseq = nseq;
+            for (uint32_t i = 0; i < nseq; ++i) ap.tiles += (seqs[i].count * H + 127) / 128;
             RUN("latent_attention", (size_t)rows * H * rank * 8, k::latent_attention(s, ap));
         }
         {   // the head's value projection on the weighted latent sum: attn[r, h, :] = W_up_v[h] ctx[r, h, :]

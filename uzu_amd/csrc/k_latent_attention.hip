@@ -8,6 +8,7 @@
 //
 // The summation order over the keys depends on the row's position and the window only, so a row's result is the same whatever else the pass carries.
 #include "device_utils.h"
+#include "gemm_convert.h"
 #include "kernels_stream32.h"
 
 namespace uzu {
@@ -87,7 +88,158 @@ __global__ void __launch_bounds__(256) latent_attention_rows_kernel(LatentAttent
     }
 }
 
+// Tiled form on the bf16 matrix cores (bf16 cache).  An ITEM is a (row, head) pair of one sequence, items numbered row-major; a wave owns 32 consecutive
+// items, a workgroup four such tiles -- with 16 heads that is 8 neighbouring rows, whose windows overlap almost entirely, so a 32-key block of latents is
+// staged once in LDS for 128 items.  Everything is computed transposed so that a lane owns one item:
+//   S^T = C Q^T    A = the block's latent rows [key][rank] from LDS, B = the item's query fragments (registers, bf16 of the f32 latent query);
+//                  the result gives a lane 16 key scores of ITS item, so the running maximum / sum are per-lane scalars (one exchange with lane ^ 32);
+//   O^T += C^T P^T A = the block transposed [rank][key] from LDS, B = those 16 weights, fed as hi + lo bf16 (16 significant bits: the weights stay f32 up
+//                  to the product); the accumulator columns are again "this lane's item": rescaling and the final 1 / l are per-lane multiplies.
+// The k order inside an MFMA only has to agree between A and B: for O^T the lane's keys are taken in the order the S^T result already holds them.
+// Scores are scaled and masked in f32 behind the MFMA; the sink enters as the initial maximum with weight 1 in the denominator.
+template <int NB> // rank padded to RP = 32 NB
+__global__ void __launch_bounds__(256) latent_attention_mfma_kernel(LatentAttentionParams p) {
+    constexpr int RP = 32 * NB, CP = RP * 2 + 16, TP = 80, VEC = RP / 8;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    uint8_t* s_c = smem;            // [32 keys][CP bytes]
+    uint8_t* s_ct = smem + 32 * CP; // [RP][TP bytes]: 32 keys + pad
+    uint32_t wg = blockIdx.x, q = 0;
+    SeqSpan sp{0, 0, 0};
+    for (;; ++q) {
+        if (q >= p.nseq) return;
+        sp = p.spans[q];
+        const uint32_t n = (sp.count * p.heads + 127) / 128;
+        if (wg < n) break;
+        wg -= n;
+    }
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
+    const uint32_t items = sp.count * p.heads;
+    auto row_lo = [&](uint32_t t) { return (p.window && t + 1 > p.window) ? t + 1 - p.window : 0u; };
+    // this lane's item
+    const uint32_t g = wg * 128 + wave * 32 + l32;
+    const bool valid = g < items;
+    const uint32_t gi = valid ? g : items - 1;
+    const uint32_t row = gi / p.heads, head = gi % p.heads;
+    const uint32_t t = sp.start + row, lo = row_lo(t);
+    // key ranges of the workgroup and of this wave
+    const uint32_t g_last = (wg * 128 + 128 < items ? wg * 128 + 128 : items) - 1;
+    const uint32_t kmin = row_lo(sp.start + wg * 128 / p.heads), kmax = sp.start + g_last / p.heads;
+    const uint32_t w_first = wg * 128 + wave * 32;
+    const bool wave_on = w_first < items;
+    const uint32_t w_last = (w_first + 32 < items ? w_first + 32 : items) - 1;
+    const uint32_t wave_lo = wave_on ? row_lo(sp.start + w_first / p.heads) : 0, wave_hi = wave_on ? sp.start + w_last / p.heads : 0;
+
+    u32x4_t qf[2 * NB];
+    {
+        const float* qrow = p.qlat + ((size_t)(sp.row0 + row) * p.heads + head) * p.rank;
+#pragma unroll
+        for (int s = 0; s < 2 * NB; ++s) {
+            const uint32_t k0 = s * 16 + half * 8;
+            u32x4_t f{0u, 0u, 0u, 0u};
+            if (valid && k0 < p.rank) { // rank % 8 == 0: a fragment is inside the row or outside it
+                const f32x4_v a = *(const f32x4_v*)(qrow + k0), b = *(const f32x4_v*)(qrow + k0 + 4);
+                f.x = (uint32_t)f32_to_bf16(a.x) | ((uint32_t)f32_to_bf16(a.y) << 16), f.y = (uint32_t)f32_to_bf16(a.z) | ((uint32_t)f32_to_bf16(a.w) << 16);
+                f.z = (uint32_t)f32_to_bf16(b.x) | ((uint32_t)f32_to_bf16(b.y) << 16), f.w = (uint32_t)f32_to_bf16(b.z) | ((uint32_t)f32_to_bf16(b.w) << 16);
+            }
+            qf[s] = f;
+        }
+    }
+    float m_run = p.sinks ? p.sinks[head] : -1.0e30f;
+    float l_run = p.sinks ? 1.0f : 0.0f;
+    f32x16_t o[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[b][r] = 0.0f;
+    const uint8_t* cache = (const uint8_t*)p.caches[q];
+
+    for (uint32_t kb = kmin; kb <= kmax; kb += 32) {
+        __syncthreads(); // the block before has been read
+        for (uint32_t v = tid; v < 32 * VEC; v += 256) {
+            const uint32_t key = v / VEC, e0 = (v % VEC) * 8, kk = kb + key;
+            u32x4_v val{0u, 0u, 0u, 0u};
+            if (kk <= kmax && e0 < p.rank) val = *(const u32x4_v*)(cache + ((size_t)kk * p.rank + e0) * 2);
+            *(u32x4_v*)(s_c + key * CP + e0 * 2) = val;
+            const uint32_t w[4] = {val.x, val.y, val.z, val.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                *(uint16_t*)(s_ct + (e0 + 2 * e) * TP + key * 2) = (uint16_t)(w[e] & 0xFFFFu);
+                *(uint16_t*)(s_ct + (e0 + 2 * e + 1) * TP + key * 2) = (uint16_t)(w[e] >> 16);
+            }
+        }
+        __syncthreads();
+        if (!wave_on || kb > wave_hi || kb + 31 < wave_lo) continue; // (wave-uniform; the barriers above are reached by every wave)
+        f32x16_t st;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) st[r] = 0.0f;
+#pragma unroll
+        for (int s = 0; s < 2 * NB; ++s) {
+            const u32x4_t a = *(const u32x4_t*)(s_c + l32 * CP + (s * 16 + half * 8) * 2);
+            st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, qf[s]), st, 0, 0, 0);
+        }
+        float mx = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const uint32_t key = kb + (r & 3) + 8 * (r >> 2) + 4 * half;
+            const bool ok = valid && key >= lo && key <= t;
+            st[r] = ok ? st[r] * p.scale : -INFINITY;
+            mx = fmaxf(mx, st[r]);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m_run, mx);
+        const float corr = fast_exp(m_run - m_new);
+        float psum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            st[r] = fast_exp(st[r] - m_new); // masked: exp(-inf) = 0
+            psum += st[r];
+        }
+        psum += __shfl_xor(psum, 32, 64);
+        l_run = fmaf(l_run, corr, psum);
+        m_run = m_new;
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[b][r] *= corr;
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+            u32x4_t hi, lw;
+            uint32_t hw[4], lwv[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float p0 = st[8 * s2 + 2 * e], p1 = st[8 * s2 + 2 * e + 1];
+                const uint16_t h0 = f32_to_bf16(p0), h1 = f32_to_bf16(p1);
+                const uint16_t l0 = f32_to_bf16(p0 - bf16_to_f32(h0)), l1 = f32_to_bf16(p1 - bf16_to_f32(h1));
+                hw[e] = (uint32_t)h0 | ((uint32_t)h1 << 16), lwv[e] = (uint32_t)l0 | ((uint32_t)l1 << 16);
+            }
+            hi = u32x4_t{hw[0], hw[1], hw[2], hw[3]}, lw = u32x4_t{lwv[0], lwv[1], lwv[2], lwv[3]};
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                const uint8_t* cr = s_ct + (b * 32 + l32) * TP + (16 * s2 + 4 * half) * 2;
+                const u32x2_v c0 = *(const u32x2_v*)cr, c1 = *(const u32x2_v*)(cr + 16);
+                const u32x4_t cf{c0.x, c0.y, c1.x, c1.y};
+                o[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, cf), __builtin_bit_cast(bf16x8_t, hi), o[b], 0, 0, 0);
+                o[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, cf), __builtin_bit_cast(bf16x8_t, lw), o[b], 0, 0, 0);
+            }
+        }
+    }
+    if (!valid) return;
+    const float inv = 1.0f / l_run;
+    float* out = p.out + ((size_t)(sp.row0 + row) * p.heads + head) * p.rank;
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+            const uint32_t col = b * 32 + 8 * g4 + 4 * half;
+            if (col < p.rank) *(f32x4_v*)(out + col) = f32x4_v{o[b][4 * g4] * inv, o[b][4 * g4 + 1] * inv, o[b][4 * g4 + 2] * inv, o[b][4 * g4 + 3] * inv};
+        }
+}
+
 } // namespace
+
+bool latent_attention_tiled_supported(const LatentAttentionParams& p) {
+    return p.cache_bf16 && p.rank % 8 == 0 && p.rank <= 256 && p.nseq > 0 && p.tiles > 0 && (uintptr_t)p.qlat % 16 == 0 && (uintptr_t)p.out % 16 == 0;
+}
 
 uzu_status latent_norm_append(hipStream_t s, const float* x, const float* scales, float eps, void* const* caches, uint32_t cache_bf16, const SeqSpan* spans,
                               const uint32_t* row_seq, uint32_t rows, uint32_t rank) {
@@ -101,6 +253,18 @@ uzu_status latent_attention(hipStream_t s, const LatentAttentionParams& p) {
     if (!p.rows) return UZU_OK;
     UZU_REQUIRE(p.qlat && p.out && p.caches && p.spans && p.row_seq && p.heads && p.rank, "latent_attention: null argument");
     UZU_UNSUPPORTED(p.rank > kLatentMaxRank, "latent_attention: latent rank %u above %u", p.rank, kLatentMaxRank);
+    UZU_UNSUPPORTED(p.form == 2 && !latent_attention_tiled_supported(p), "latent_attention: the tiled form takes a bf16 cache, rank %% 8 == 0, rank <= 256");
+    if (p.form != 1 && latent_attention_tiled_supported(p)) {
+        static LdsLimit lim4, lim8;
+        if (p.rank <= 128) {
+            const size_t lds = 32 * (128 * 2 + 16) + 128 * 80;
+            raise_lds_limit(lim4, (const void*)latent_attention_mfma_kernel<4>, lds);
+            return launch_check([&] { hipLaunchKernelGGL(latent_attention_mfma_kernel<4>, dim3(p.tiles), dim3(256), lds, s, p); }, "latent_attention_mfma");
+        }
+        const size_t lds = 32 * (256 * 2 + 16) + 256 * 80;
+        raise_lds_limit(lim8, (const void*)latent_attention_mfma_kernel<8>, lds);
+        return launch_check([&] { hipLaunchKernelGGL(latent_attention_mfma_kernel<8>, dim3(p.tiles), dim3(256), lds, s, p); }, "latent_attention_mfma");
+    }
     const uint32_t items = p.rows * p.heads;
     const dim3 grid((items + 3) / 4), block(256);
     const uint32_t nt = (p.rank + 63) / 64;

@@ -96,7 +96,11 @@ struct LatentAttentionParams {
     const uint32_t* row_seq;
     uint32_t rows, heads, rank, window;
     float scale;
+    uint32_t form; // 0: chosen by shape; 1: the simple form (a wave per row and head, keys one after the other); 2: the tiled form
+    uint32_t nseq;  // entries of `spans`
+    uint32_t tiles; // sum over the sequences of ceil(count * heads / 128): the tiled form's workgroups (the caller knows the counts)
 };
+bool latent_attention_tiled_supported(const LatentAttentionParams& p);
 uzu_status latent_attention(hipStream_t s, const LatentAttentionParams& p);
 constexpr uint32_t kLatentMaxRank = 1024;
 

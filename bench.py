@@ -56,6 +56,10 @@ def parse_args():
                     help="BASELINE.json configs[1..4]: c2 (default, the headline) Qwen3.5-0.8B int4 ctx-2048 decode; c3 Llama-3-8B int4, 4k prefill x 8 "
                          "sequences in batched passes (prefill tokens/s, MFMA roofline); c4 Llama-3-8B int8 decode (TP = --gpus); c5 Qwen3-14B-class int4 at "
                          "ctx 8192, one sequence decoding while another is prefilled (TP = --gpus)")
+    ap.add_argument("--design", choices=["", "lazolix"], default="", help="side runs of a design outside BASELINE.json (never the headline): `lazolix` times prefill, "
+                    "chained decode and batched decode of the f32-stream design at layer sizes of real models (random weights), beside the closest "
+                    "bf16-stream model of the engine at equal sizes (windowed attention with sinks + int4 dense / bf16 expert MLPs)")
+    ap.add_argument("--design-sizes", default="w1024,w2048", help="--design: comma-separated size presets")
     ap.add_argument("--sequences", type=int, default=8, help="c3: sequences per batched prefill pass")
     ap.add_argument("--prompt", type=int, default=4096, help="c3: prompt tokens per sequence")
     args = ap.parse_args()
@@ -459,8 +463,100 @@ def spawn_ranks(n):
     sys.exit(subprocess.call(cmd, env=env))
 
 
+LAZOLIX_SIZES = {  # layer sizes of real models: width, heads x (dim, vdim), latent rank, window, dense ff, experts x ff
+    "w1024": dict(width=1024, heads=8, dim=128, vdim=128, rank=256, window=1024, ff=4096, experts=8, top=2, eff=1024, identity=1, layers=4, vocab=32768),
+    "w2048": dict(width=2048, heads=16, dim=128, vdim=128, rank=256, window=1024, ff=8192, experts=8, top=2, eff=2048, identity=1, layers=4, vocab=32768),
+}
+
+
+def bench_lazolix(args):
+    """Prefill / decode throughput of Lazolix models (dense and expert MLPs) and of the closest bf16-stream model at the same sizes.  One JSON line."""
+    import tempfile
+    from uzu_amd import desc as D, lazolix, loader, synthetic as S
+    from uzu_amd.backend import Context
+    from uzu_amd.engine import MODEL_BATCH, MODEL_DEFAULT, HipModel
+    ctx = Context.new(0)
+    prompt_len, steps, warm, nbatch = 2048, max(8, min(args.steps, 128)), max(2, min(args.warmup, 8)), 8
+    out = {"metric": "lazolix_side_run", "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16 products, f32 stream", "data": "synthetic (random weights, synthetic token ids)",
+           "prompt_tokens": prompt_len, "decode_steps": steps, "batched_decode_sequences": nbatch, "sizes": {}}
+
+    def timed(fn, reps=3):
+        fn()
+        ctx.synchronize()
+        best = 1e30
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            fn()
+            ctx.synchronize()
+            best = min(best, time.perf_counter() - t0)
+        return best
+
+    for size in [s for s in args.design_sizes.split(",") if s]:
+        z = LAZOLIX_SIZES[size]
+        rec = {}
+        prompt = S.synthetic_prompt(prompt_len, z["vocab"]).astype(np.uint32)
+        for kind in ("dense", "moe"):
+            mlp = lazolix.dense_mlp(z["ff"]) if kind == "dense" else lazolix.moe_mlp(z["experts"], z["top"], z["eff"], z["identity"])
+            layers = [lazolix.layer_config(z["heads"], z["dim"], z["vdim"], z["rank"], z["window"], kv_from=(l - 1 if l % 2 else None), mlp=mlp) for l in range(z["layers"])]
+            cfg = {"vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-6}, "layers": layers}
+            with tempfile.TemporaryDirectory() as tmp:
+                lazolix.save(tmp, cfg, lazolix.random_tensors(cfg, seed=1))
+                bundle = loader.load_model_dir(tmp, max_context_length=prompt_len + steps + warm + 64)
+            m = HipModel(ctx, bundle, MODEL_BATCH(nbatch))
+
+            def prefill():
+                m.reset()
+                m.prefill(prompt)
+            t_prefill = timed(prefill)
+            m.decode(warm)
+            t0 = time.perf_counter()
+            m.decode(steps)
+            ctx.synchronize()
+            t_decode = time.perf_counter() - t0
+            states = [m.new_state() for _ in range(nbatch)]
+            m.step_batch(states, [list(prompt)] * nbatch, None)
+            step = lambda: m.step_batch(states, [[7]] * nbatch, None, sample=True)
+            t_batch = timed(step, reps=8)
+            rec["lazolix_" + kind] = {"prefill_tokens_per_s": round(prompt_len / t_prefill, 1), "prefill_tflops": round(bundle.prefill_flops(prompt_len) / t_prefill / 1e12, 2),
+                                      "decode_tokens_per_s": round(steps / t_decode, 1), "decode_us_per_token": round(t_decode / steps * 1e6, 1),
+                                      "decode_launches": m.decode_launch_count, "decode_gbps": round(bundle.decode_bytes_per_token(prompt_len) * steps / t_decode / 1e9, 1),
+                                      "batched_decode_tokens_per_s": round(nbatch / t_batch, 1), "weight_bytes": m.weight_bytes}
+            for st in states:
+                st.close()
+            m.close()
+            # the closest bf16-stream model: windowed attention with sinks, same width / heads / head width / layers / vocabulary; int4 g128 dense MLP of the same
+            # hidden width, or bf16 experts of the same count and width
+            ccfg = S.ModelConfig(name=f"closest-{size}-{kind}", vocab_size=z["vocab"], model_dim=z["width"], hidden_dim=z["ff"], layer_kinds=[D.MIXER_ATTENTION] * z["layers"],
+                                 num_heads=z["heads"], num_groups=z["heads"], head_dim=z["dim"], rope=D.RopeConfig(kind=D.ROPE_UNSCALED, head_dim=z["dim"], max_sequence_length=8192, base=10000.0),
+                                 sliding_windows=[z["window"]] * z["layers"], sinks=True, bits=4, group_size=128, tied_embeddings=True,
+                                 max_context_length=prompt_len + steps + warm + 64, seed=5,
+                                 **({"moe_experts": z["experts"], "moe_active": z["top"], "moe_hidden": z["eff"]} if kind == "moe" else {}))
+            cb = S.build_model(ccfg)
+            cm = HipModel(ctx, cb, MODEL_DEFAULT)
+
+            def cprefill():
+                cm.reset()
+                cm.prefill(prompt)
+            ct_prefill = timed(cprefill)
+            cm.decode(warm)
+            t0 = time.perf_counter()
+            cm.decode(steps)
+            ctx.synchronize()
+            ct_decode = time.perf_counter() - t0
+            rec["closest_" + kind] = {"prefill_tokens_per_s": round(prompt_len / ct_prefill, 1), "prefill_tflops": round(cb.prefill_flops(prompt_len) / ct_prefill / 1e12, 2),
+                                      "decode_tokens_per_s": round(steps / ct_decode, 1), "decode_us_per_token": round(ct_decode / steps * 1e6, 1),
+                                      "decode_launches": cm.decode_launch_count, "decode_gbps": round(cb.decode_bytes_per_token(prompt_len) * steps / ct_decode / 1e9, 1),
+                                      "weight_bytes": cm.weight_bytes}
+            cm.close()
+        out["sizes"][size] = {"shape": z, **rec}
+    ctx.close()
+    print(json.dumps(out), flush=True)
+
+
 def main():
     args = parse_args()
+    if args.design == "lazolix":
+        return bench_lazolix(args)
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ and not args.force_dist:
         spawn_ranks(args.gpus)
     if args.config == "c3":

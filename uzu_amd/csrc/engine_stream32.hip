@@ -57,7 +57,8 @@ void state_set_length(uzu_hip_model* m, uzu_hip_state* st, uint32_t len) {
     if (m->bound == st) m->context_length = len;
 }
 
-__global__ void s32_commit_kernel(uint32_t* ctx_len, uint32_t* tokens, const uint32_t* out_token, uint32_t* sampled, uint32_t count, uint32_t has_token) {
+// `span` (optional): the device-side span of a one-sequence decode step moves on with the context, so the next step needs nothing from the host
+__global__ void s32_commit_kernel(uint32_t* ctx_len, uint32_t* tokens, const uint32_t* out_token, uint32_t* sampled, uint32_t count, uint32_t has_token, k::SeqSpan* span) {
     const uint32_t len = *ctx_len;
     if (has_token) {
         const uint32_t t = *out_token;
@@ -65,6 +66,7 @@ __global__ void s32_commit_kernel(uint32_t* ctx_len, uint32_t* tokens, const uin
         tokens[0] = t;
     }
     *ctx_len = len + count;
+    if (span) span->start = len + count;
 }
 
 uzu_status need_f32(uzu_hip_model* m, size_t floats, float** out) {
@@ -94,15 +96,11 @@ void run_linear(Enc& e, const k::LinearF32Params& p) {
     e.run(r, variant, k::linear_f32_bytes(p));
 }
 
-// One pass over `seqs` (rows = sum of their counts, <= max_rows; token ids on the device, row-major in sequence order).  `out_rows`: rows of the pass whose
-// logits are wanted, in order; they land in S.logits [out_rows.size()][vocab] f32.  Does not move the sequences' context lengths.
-uzu_status s32_pass(uzu_hip_model* m, const std::vector<PassSeq>& seqs, const uint32_t* d_tokens, const std::vector<uint32_t>& out_rows) {
+// The tables of a pass over `seqs`: spans, row -> sequence, per-layer cache / shift-state pointers, the rows whose logits are wanted.
+uzu_status s32_upload_tables(uzu_hip_model* m, const std::vector<PassSeq>& seqs, const std::vector<uint32_t>& out_rows) {
     Stream32& S = *m->s32;
     hipStream_t s = m->ctx->stream;
-    Enc e{m, s};
-    e.prof = (std::vector<ProfEntry>*)m->prof_sink;
-    m->launches = 0;
-    const uint32_t d = m->d.model_dim, nl = m->d.num_layers, nseq = (uint32_t)seqs.size();
+    const uint32_t nl = m->d.num_layers, nseq = (uint32_t)seqs.size();
     UZU_REQUIRE(nseq > 0 && nseq <= S.max_seqs, "engine: a pass of %u sequences (the model carries at most %u)", nseq, S.max_seqs);
     std::vector<k::SeqSpan> spans(nseq);
     std::vector<uint32_t> row_seq;
@@ -130,7 +128,21 @@ uzu_status s32_pass(uzu_hip_model* m, const std::vector<PassSeq>& seqs, const ui
     HIPCHK(hipMemcpyAsync(S.d_cache_ptrs, cache_ptrs.data(), cache_ptrs.size() * sizeof(void*), hipMemcpyHostToDevice, s));
     HIPCHK(hipMemcpyAsync(S.d_shift_ptrs, shift_ptrs.data(), shift_ptrs.size() * sizeof(float*), hipMemcpyHostToDevice, s));
     if (!out_rows.empty()) HIPCHK(hipMemcpyAsync(S.d_out_rows, out_rows.data(), out_rows.size() * 4, hipMemcpyHostToDevice, s));
+    return UZU_OK;
+}
 
+// The launches of one pass (tables uploaded before): rows = sum of the sequences' counts (<= max_rows), token ids on the device, row-major in sequence order;
+// n_out rows (S.d_out_rows) get logits in S.logits [n_out][vocab] f32.  Nothing here depends on the sequences' positions -- the kernels read them from the
+// device-side spans -- so a one-token step can be captured once and replayed.  Does not move the sequences' context lengths.
+uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, const uint32_t* d_tokens, uint32_t n_out) {
+    Stream32& S = *m->s32;
+    hipStream_t s = m->ctx->stream;
+    Enc e{m, s};
+    e.prof = (std::vector<ProfEntry>*)m->prof_sink;
+    m->launches = 0;
+    const uint32_t d = m->d.model_dim, nl = m->d.num_layers, nseq = (uint32_t)counts.size();
+    uint32_t rows = 0;
+    for (uint32_t c : counts) rows += c;
     const size_t slot_stride = (size_t)S.max_rows * d;
     const uint32_t bf = S.full_f32 ? 0u : 1u;
     RUN("embed_rows_f32", (size_t)rows * d * 6, k::embed_rows_f32(s, d_tokens, (const uint16_t*)m->embedding.w, S.slots, rows, m->d.vocab_size, d));
@@ -166,7 +178,7 @@ uzu_status s32_pass(uzu_hip_model* m, const std::vector<PassSeq>& seqs, const ui
             ap.rows = rows, ap.heads = H, ap.rank = rank, ap.window = h.sliding_window_size;
             ap.scale = h.attention_scale != 0.0f ? h.attention_scale : 1.0f / sqrtf((float)hd);
             ap.nseq = nseq;
-            for (uint32_t i = 0; i < nseq; ++i) ap.tiles += (seqs[i].count * H + 127) / 128;
+            for (uint32_t i = 0; i < nseq; ++i) ap.tiles += (counts[i] * H + 127) / 128;
             RUN("latent_attention", (size_t)rows * H * rank * 8, k::latent_attention(s, ap));
         }
         {   // the head's value projection on the weighted latent sum: attn[r, h, :] = W_up_v[h] ctx[r, h, :]
@@ -211,8 +223,7 @@ uzu_status s32_pass(uzu_hip_model* m, const std::vector<PassSeq>& seqs, const ui
     }
     S.tap_rows = rows;
     S.last_logit_rows = 0;
-    if (!out_rows.empty()) {
-        const uint32_t n_out = (uint32_t)out_rows.size();
+    if (n_out) {
         k::DynTanhParams np{};
         np.x = cur, np.out = S.out_normed, np.scales = m->output_norm.scales, np.biases = m->output_norm.biases, np.alpha = S.alpha_out, np.row_index = S.d_out_rows;
         np.rows = n_out, np.d = d;
@@ -229,10 +240,27 @@ uzu_status s32_pass(uzu_hip_model* m, const std::vector<PassSeq>& seqs, const ui
     return UZU_OK;
 }
 
+uzu_status s32_pass(uzu_hip_model* m, const std::vector<PassSeq>& seqs, const uint32_t* d_tokens, const std::vector<uint32_t>& out_rows) {
+    UZU_PROPAGATE(s32_upload_tables(m, seqs, out_rows));
+    std::vector<uint32_t> counts;
+    for (const PassSeq& q : seqs) counts.push_back(q.count);
+    return s32_encode(m, counts, d_tokens, (uint32_t)out_rows.size());
+}
+
 uzu_status ensure_logits(uzu_hip_model* m, size_t rows) {
     Stream32& S = *m->s32;
     if (rows <= S.logit_rows) return UZU_OK;
     HIPCHK(hipStreamSynchronize(m->ctx->stream));
+    // captured decode steps carry the old block's address: every state's graph goes (it is rebuilt at that state's next decode)
+    auto drop = [](hipGraphExec_t& g) {
+        if (g) (void)hipGraphExecDestroy(g);
+        g = nullptr;
+    };
+    drop(m->graph_single);
+    if (m->state0 && m->state0 != m->bound) drop(m->state0->graph_single);
+    for (uzu_hip_state* u : m->user_states)
+        if (u != m->bound) drop(u->graph_single);
+    if (m->bound) m->bound->graph_single = nullptr;
     if (S.logits) dev_free(m, S.logits);
     S.logits = nullptr, S.logit_rows = 0;
     size_t want = rows < 16 ? 16 : rows;
@@ -243,7 +271,7 @@ uzu_status ensure_logits(uzu_hip_model* m, size_t rows) {
 }
 
 // sample from row `logit_row` of the last pass's logits into st's control block and advance it by `count`
-uzu_status sample_commit(uzu_hip_model* m, uzu_hip_state* st, uint32_t logit_row, uint32_t count, bool sample) {
+uzu_status sample_commit(uzu_hip_model* m, uzu_hip_state* st, uint32_t logit_row, uint32_t count, bool sample, k::SeqSpan* span = nullptr) {
     Stream32& S = *m->s32;
     hipStream_t s = m->ctx->stream;
     Enc e{m, s};
@@ -259,7 +287,7 @@ uzu_status sample_commit(uzu_hip_model* m, uzu_hip_state* st, uint32_t logit_row
         }
     }
     if (e.st != UZU_OK) return e.st;
-    hipLaunchKernelGGL(s32_commit_kernel, dim3(1), dim3(1), 0, s, st->d_ctx_len, st->d_tokens, st->d_out_token, st->d_sampled, count, sample ? 1u : 0u);
+    hipLaunchKernelGGL(s32_commit_kernel, dim3(1), dim3(1), 0, s, st->d_ctx_len, st->d_tokens, st->d_out_token, st->d_sampled, count, sample ? 1u : 0u, span);
     ++m->launches;
     return UZU_OK;
 }
@@ -538,11 +566,38 @@ uzu_status s32_decode_enqueue(uzu_hip_model* m, uint32_t steps) {
     uzu_hip_state* st = m->bound;
     UZU_REQUIRE(m->context_length + steps <= m->d.max_context_length, "model_decode: %u + %u tokens exceed max_context_length %u", m->context_length, steps, m->d.max_context_length);
     UZU_PROPAGATE(ensure_logits(m, 1));
-    const std::vector<uint32_t> out_rows{0};
+    Stream32& S = *m->s32;
+    hipStream_t s = m->ctx->stream;
+    // the tables once (the model's table block serves whichever state steps; the span moves on the device with every commit)
+    UZU_PROPAGATE(s32_upload_tables(m, {{st, 1, m->context_length}}, {0}));
+    const std::vector<uint32_t> one{1};
+    const bool graph = !(m->flags & (UZU_MODEL_NO_GRAPH | UZU_MODEL_DEBUG_TAPS));
+    if (graph && m->graph_epoch != m->sampling_epoch) { // the captured step bakes the sampling kernels in
+        if (m->graph_single) (void)hipGraphExecDestroy(m->graph_single);
+        m->graph_single = nullptr, m->graph_epoch = m->sampling_epoch;
+    }
+    if (graph && !m->graph_single) { // one decode step of THIS state (its token / cache / control-block pointers) as a hipGraph
+        HIPCHK(hipStreamSynchronize(s));
+        HIPCHK(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal));
+        uzu_status r = s32_encode(m, one, st->d_tokens, 1);
+        if (r == UZU_OK) r = sample_commit(m, st, 0, 1, true, S.d_spans);
+        hipGraph_t g = nullptr;
+        const hipError_t ce = hipStreamEndCapture(s, &g);
+        if (r != UZU_OK || ce != hipSuccess) {
+            if (g) (void)hipGraphDestroy(g);
+            if (r == UZU_OK) set_error("engine: decode graph capture failed: %s", hipGetErrorString(ce));
+            return r != UZU_OK ? r : UZU_ERR_HIP;
+        }
+        HIPCHK(hipGraphInstantiate(&m->graph_single, g, nullptr, nullptr, 0));
+        HIPCHK(hipGraphDestroy(g));
+    }
     for (uint32_t i = 0; i < steps; ++i) {
-        const std::vector<PassSeq> pass{{st, 1, m->context_length}};
-        UZU_PROPAGATE(s32_pass(m, pass, st->d_tokens, out_rows));
-        UZU_PROPAGATE(sample_commit(m, st, 0, 1, true));
+        if (graph) {
+            HIPCHK(hipGraphLaunch(m->graph_single, s));
+        } else {
+            UZU_PROPAGATE(s32_encode(m, one, st->d_tokens, 1));
+            UZU_PROPAGATE(sample_commit(m, st, 0, 1, true, S.d_spans));
+        }
         state_set_length(m, st, m->context_length + 1);
     }
     return UZU_OK;

@@ -160,7 +160,7 @@ uzu_status uzu_hip_s32_latent_norm_append(uzu_hip_context* ctx, const float* x, 
 }
 
 // qlat / out [rows][heads * rank] for positions start .. start + rows - 1; cache f32 [(start + rows)][rank] (rounded to bf16 here when cache_bf16).
-// form 0: the engine's choice for the shape; 1: the simple form (a wave per row and head); 2: the tiled form
+// form 0: the engine's choice for the shape; 1: the simple form (a wave per row and head); 2: the tiled form; 3: the tiled form with split keys + merge
 uzu_status uzu_hip_s32_latent_attention(uzu_hip_context* ctx, const float* qlat, const float* cache, const float* sinks, float* out, uint32_t rows, uint32_t start, uint32_t heads,
                                         uint32_t rank, uint32_t window, float scale, uint32_t cache_bf16, uint32_t form) {
     UZU_REQUIRE(ctx && qlat && cache && out, "s32_latent_attention: null argument");
@@ -188,6 +188,13 @@ uzu_status uzu_hip_s32_latent_attention(uzu_hip_context* ctx, const float* qlat,
     k::LatentAttentionParams p{};
     p.qlat = dq, p.out = dout, p.caches = dcp, p.cache_bf16 = cache_bf16, p.sinks = dsink, p.spans = spans, p.row_seq = row_seq;
     p.rows = rows, p.heads = heads, p.rank = rank, p.window = window, p.scale = scale, p.form = form, p.nseq = 1, p.tiles = (rows * heads + 127) / 128;
+    float* ws = nullptr;
+    if (form == 3) { // the tiled form with its key blocks split over workgroups + the merge launch
+        p.form = 2, p.splits = 5;
+        p.split_ws_bytes = k::latent_attention_split_ws_bytes(rows, heads, rank, p.splits);
+        UZU_PROPAGATE(S.up((const float*)nullptr, p.split_ws_bytes / 4, &ws));
+        p.split_ws = ws;
+    }
     UZU_PROPAGATE(k::latent_attention(ctx->stream, p));
     UZU_PROPAGATE(finish(ctx));
     UZU_HIP_TRY(hipMemcpy(out, dout, (size_t)rows * heads * rank * 4, hipMemcpyDeviceToHost));
@@ -217,8 +224,24 @@ uzu_status uzu_hip_s32_moe(uzu_hip_context* ctx, const float* x, const uint16_t*
     UZU_PROPAGATE(S.up((const float*)nullptr, (size_t)rows * top * (ff ? ff : 1), &dh));
     UZU_PROPAGATE(S.up((const int32_t*)nullptr, (size_t)rows * top, &dids));
     UZU_PROPAGATE(k::moe_route_scores(ctx->stream, dx, dr, dsb, dids, dwt, rows, d, routed + identity, top));
-    UZU_PROPAGATE(k::moe_experts_gate_up(ctx->stream, dx, dids, d13, dh, rows, d, ff, routed, top, bf16_products));
-    UZU_PROPAGATE(k::moe_experts_down_combine(ctx->stream, dh, dx, dids, dwt, d2, dres, dy, rows, d, ff, routed, top, bf16_products));
+    if (bf16_products == 2) { // bf16 products through the grouped matrix-core form
+        k::MoeGroupedParams gp{};
+        uint32_t *perm, *slot_pos, *offsets, *cursor;
+        float *y1, *y2;
+        UZU_PROPAGATE(S.up((const float*)nullptr, (size_t)rows * top * 2 * ff, &y1));
+        UZU_PROPAGATE(S.up((const float*)nullptr, (size_t)rows * top * d, &y2));
+        UZU_PROPAGATE(S.up((const uint32_t*)nullptr, (size_t)rows * top, &perm));
+        UZU_PROPAGATE(S.up((const uint32_t*)nullptr, (size_t)rows * top, &slot_pos));
+        UZU_PROPAGATE(S.up((const uint32_t*)nullptr, (size_t)routed + 1, &offsets));
+        UZU_PROPAGATE(S.up((const uint32_t*)nullptr, (size_t)routed + 1, &cursor));
+        gp.x = dx, gp.ids = dids, gp.weights = dwt, gp.w13 = d13, gp.w2 = d2, gp.residual = dres, gp.y = dy, gp.y1 = y1, gp.hidden = dh, gp.y2 = y2;
+        gp.perm = perm, gp.slot_pos = slot_pos, gp.offsets = offsets, gp.cursor = cursor, gp.rows = rows, gp.d = d, gp.ff = ff, gp.routed = routed, gp.top = top;
+        UZU_UNSUPPORTED(!k::moe_experts_grouped_supported(gp), "s32_moe: the grouped form does not take this shape");
+        UZU_PROPAGATE(k::moe_experts_grouped(ctx->stream, gp));
+    } else {
+        UZU_PROPAGATE(k::moe_experts_gate_up(ctx->stream, dx, dids, d13, dh, rows, d, ff, routed, top, bf16_products));
+        UZU_PROPAGATE(k::moe_experts_down_combine(ctx->stream, dh, dx, dids, dwt, d2, dres, dy, rows, d, ff, routed, top, bf16_products));
+    }
     UZU_PROPAGATE(finish(ctx));
     UZU_HIP_TRY(hipMemcpy(y, dy, (size_t)rows * d * 4, hipMemcpyDeviceToHost));
     if (ids_out) UZU_HIP_TRY(hipMemcpy(ids_out, dids, (size_t)rows * top * 4, hipMemcpyDeviceToHost));

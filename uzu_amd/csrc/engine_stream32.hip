@@ -30,6 +30,8 @@ struct Stream32 {
     float *slots = nullptr, *xin = nullptr, *normed = nullptr, *q = nullptr, *ckv = nullptr, *qlat = nullptr, *ctx = nullptr, *attn = nullptr, *hid = nullptr;
     int32_t* moe_ids = nullptr;
     float* moe_w = nullptr;
+    float *moe_y1 = nullptr, *moe_y2 = nullptr; // grouped expert form: [max_rows * top][2 ff] and [max_rows * top][d]
+    uint32_t *moe_perm = nullptr, *moe_slot_pos = nullptr, *moe_offsets = nullptr, *moe_cursor = nullptr;
     float *out_normed = nullptr, *logits = nullptr;
     size_t logit_rows = 0;
     k::SeqSpan* d_spans = nullptr;
@@ -44,6 +46,8 @@ struct Stream32 {
     };
     std::vector<Layer> layers;
     float alpha_out = 0.f;
+    float* att_ws = nullptr; // partial sums of the key-split attention of decode-sized passes
+    size_t att_ws_bytes = 0;
     float* taps = nullptr; // UZU_MODEL_DEBUG_TAPS: f32 [layers][max_rows][d], what each layer handed on in the last pass
     uint32_t tap_rows = 0;
     uint32_t last_logit_rows = 0; // rows of `logits` the last pass produced
@@ -178,6 +182,9 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
             ap.rows = rows, ap.heads = H, ap.rank = rank, ap.window = h.sliding_window_size;
             ap.scale = h.attention_scale != 0.0f ? h.attention_scale : 1.0f / sqrtf((float)hd);
             ap.nseq = nseq;
+            // decode-sized passes: spread a tile's key blocks over workgroups (a constant of the layer, so that a captured step stays valid as the context grows)
+            const uint32_t keys = h.sliding_window_size ? h.sliding_window_size : m->d.max_context_length;
+            if (rows <= 4 * S.max_seqs && rows * H <= 4096) ap.splits = std::min<uint32_t>(32, (keys + 31) / 32), ap.split_ws = S.att_ws, ap.split_ws_bytes = S.att_ws_bytes;
             for (uint32_t i = 0; i < nseq; ++i) ap.tiles += (counts[i] * H + 127) / 128;
             RUN("latent_attention", (size_t)rows * H * rank * 8, k::latent_attention(s, ap));
         }
@@ -201,9 +208,17 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
                 const uint32_t E = M.num_routed_experts, top = M.num_active_experts, ff = M.expert_hidden_dim;
                 RUN("moe_route_scores", (size_t)(E + M.num_identity_experts) * d * 2,
                     k::moe_route_scores(s, S.normed, L.moe.router_weights, X.selection_bias, S.moe_ids, S.moe_w, rows, d, E + M.num_identity_experts, top));
-                RUN("moe_experts_gate_up", (size_t)rows * top * 2 * ff * d * 2, k::moe_experts_gate_up(s, S.normed, S.moe_ids, L.moe.w13, S.hid, rows, d, ff, E, top, bf));
-                RUN("moe_experts_down_combine", (size_t)rows * top * ff * d * 2,
-                    k::moe_experts_down_combine(s, S.hid, S.normed, S.moe_ids, S.moe_w, L.moe.w2, slot, slot, rows, d, ff, E, top, bf));
+                k::MoeGroupedParams gp{};
+                gp.x = S.normed, gp.ids = S.moe_ids, gp.weights = S.moe_w, gp.w13 = L.moe.w13, gp.w2 = L.moe.w2, gp.residual = slot, gp.y = slot, gp.y1 = S.moe_y1, gp.hidden = S.hid;
+                gp.y2 = S.moe_y2, gp.perm = S.moe_perm, gp.slot_pos = S.moe_slot_pos, gp.offsets = S.moe_offsets, gp.cursor = S.moe_cursor;
+                gp.rows = rows, gp.d = d, gp.ff = ff, gp.routed = E, gp.top = top;
+                if (bf && k::moe_experts_grouped_supported(gp)) { // prefill-sized: buckets per expert through the matrix-core linear
+                    RUN("moe_experts_grouped", (size_t)E * 3 * ff * d * 2 + (size_t)rows * top * (3 * ff + 2 * d) * 4, k::moe_experts_grouped(s, gp));
+                } else {
+                    RUN("moe_experts_gate_up", (size_t)rows * top * 2 * ff * d * 2, k::moe_experts_gate_up(s, S.normed, S.moe_ids, L.moe.w13, S.hid, rows, d, ff, E, top, bf));
+                    RUN("moe_experts_down_combine", (size_t)rows * top * ff * d * 2,
+                        k::moe_experts_down_combine(s, S.hid, S.normed, S.moe_ids, S.moe_w, L.moe.w2, slot, slot, rows, d, ff, E, top, bf));
+                }
             } else {
                 k::LinearF32Params up = lin(S, L.up, S.normed, S.hid, rows);
                 up.act = 1;
@@ -358,7 +373,7 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
     S.max_rows = m->chunk, S.max_seqs = m->max_seqs;
     m->layers.resize(nl);
     S.layers.resize(nl);
-    uint32_t w_q = 0, w_rank = 0, w_lat = 0, w_attn = 0, w_hid = 0, w_top = 1;
+    uint32_t w_q = 0, w_rank = 0, w_lat = 0, w_attn = 0, w_hid = 0, w_top = 1, w_moe = 0, w_routed = 0;
     for (uint32_t l = 0; l < nl; ++l) {
         const uzu_layer_desc& h = desc->layers[l];
         DLayer& L = m->layers[l];
@@ -404,6 +419,7 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
                 if (M.selection_bias) TRY(upload(m, M.selection_bias, (E + M.num_identity_experts) * 4, &X.selection_bias));
                 w_hid = std::max<uint32_t>(w_hid, M.num_active_experts * M.expert_hidden_dim);
                 w_top = std::max(w_top, M.num_active_experts);
+                w_moe = std::max(w_moe, M.num_active_experts * 2 * M.expert_hidden_dim), w_routed = std::max(w_routed, M.num_routed_experts);
             } else {
                 TRY(upload_linear(m, h.up_projection, &L.up));
                 TRY(upload_linear(m, h.down_projection, &L.down));
@@ -425,6 +441,15 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
     TRY(need_f32(m, R * w_attn, &S.attn));
     TRY(need_f32(m, R * (w_hid ? w_hid : 1), &S.hid));
     TRY(need_f32(m, R * w_top, &S.moe_w));
+    if (w_moe && !S.full_f32) { // workspaces of the grouped expert form (bf16 products only)
+        void* q = nullptr;
+        TRY(need_f32(m, R * w_moe, &S.moe_y1));
+        TRY(need_f32(m, R * w_top * d, &S.moe_y2));
+        TRY(dev_alloc(m, R * w_top * 4, &q, true)); S.moe_perm = (uint32_t*)q;
+        TRY(dev_alloc(m, R * w_top * 4, &q, true)); S.moe_slot_pos = (uint32_t*)q;
+        TRY(dev_alloc(m, ((size_t)w_routed + 1) * 4, &q, true)); S.moe_offsets = (uint32_t*)q;
+        TRY(dev_alloc(m, ((size_t)w_routed + 1) * 4, &q, true)); S.moe_cursor = (uint32_t*)q;
+    }
     void* p = nullptr;
     TRY(dev_alloc(m, R * w_top * 4, &p, true)); S.moe_ids = (int32_t*)p;
     TRY(dev_alloc(m, S.max_seqs * sizeof(k::SeqSpan), &p, true)); S.d_spans = (k::SeqSpan*)p;
@@ -434,6 +459,12 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
     TRY(dev_alloc(m, (size_t)nl * S.max_seqs * sizeof(float*), &p, true)); S.d_shift_ptrs = (float**)p;
     TRY(dev_alloc(m, R * 4, &p, true)); m->batch_tokens = (uint32_t*)p;
     if (flags & UZU_MODEL_DEBUG_TAPS) TRY(need_f32(m, (size_t)nl * R * d, &S.taps));
+    {
+        uint32_t hmax = 0;
+        for (uint32_t l = 0; l < nl; ++l) hmax = std::max(hmax, desc->layers[l].num_heads);
+        S.att_ws_bytes = k::latent_attention_split_ws_bytes(std::min<uint32_t>(4 * S.max_seqs, 4096 / hmax ? 4096 / hmax : 1), hmax, 256, 32);
+        TRY(need_f32(m, S.att_ws_bytes / 4, &S.att_ws));
+    }
     TRY(dev_alloc(m, k::argmax_scratch_bytes(1), &m->argmax_scratch));
     TRY(dev_alloc(m, k::unified_sampling_scratch_bytes(1), &m->sampling_scratch));
     TRY(dev_alloc(m, 8, &p, true)); m->d_seed = (uint64_t*)p;

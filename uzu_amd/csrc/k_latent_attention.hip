@@ -97,7 +97,9 @@ __global__ void __launch_bounds__(256) latent_attention_rows_kernel(LatentAttent
 //                  to the product); the accumulator columns are again "this lane's item": rescaling and the final 1 / l are per-lane multiplies.
 // The k order inside an MFMA only has to agree between A and B: for O^T the lane's keys are taken in the order the S^T result already holds them.
 // Scores are scaled and masked in f32 behind the MFMA; the sink enters as the initial maximum with weight 1 in the denominator.
-template <int NB> // rank padded to RP = 32 NB
+// SPLIT (few items, many keys: decode steps): grid.y workgroups share an item tile's key blocks (block i goes to workgroup i mod grid.y) and leave unnormalised
+// sums with their running maximum / denominator in p.split_ws; latent_attention_merge_kernel combines them.  The sink belongs to split 0.
+template <int NB, bool SPLIT> // rank padded to RP = 32 NB
 __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(LatentAttentionParams p) {
     constexpr int RP = 32 * NB, CP = RP * 2 + 16, TP = 80, VEC = RP / 8;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -144,8 +146,9 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(LatentAttent
             qf[s] = f;
         }
     }
-    float m_run = p.sinks ? p.sinks[head] : -1.0e30f;
-    float l_run = p.sinks ? 1.0f : 0.0f;
+    const bool with_sink = p.sinks && (!SPLIT || blockIdx.y == 0);
+    float m_run = with_sink ? p.sinks[head] : -1.0e30f;
+    float l_run = with_sink ? 1.0f : 0.0f;
     f32x16_t o[NB];
 #pragma unroll
     for (int b = 0; b < NB; ++b)
@@ -153,7 +156,8 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(LatentAttent
         for (int r = 0; r < 16; ++r) o[b][r] = 0.0f;
     const uint8_t* cache = (const uint8_t*)p.caches[q];
 
-    for (uint32_t kb = kmin; kb <= kmax; kb += 32) {
+    const uint32_t kstep = SPLIT ? 32 * gridDim.y : 32;
+    for (uint32_t kb = kmin + (SPLIT ? 32 * blockIdx.y : 0); kb <= kmax; kb += kstep) {
         __syncthreads(); // the block before has been read
         for (uint32_t v = tid; v < 32 * VEC; v += 256) {
             const uint32_t key = v / VEC, e0 = (v % VEC) * 8, kk = kb + key;
@@ -224,6 +228,16 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(LatentAttent
         }
     }
     if (!valid) return;
+    if (SPLIT) {
+        float* ws = p.split_ws + (((size_t)(sp.row0 + row) * p.heads + head) * gridDim.y + blockIdx.y) * (RP + 4);
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4)
+                *(f32x4_v*)(ws + b * 32 + 8 * g4 + 4 * half) = f32x4_v{o[b][4 * g4], o[b][4 * g4 + 1], o[b][4 * g4 + 2], o[b][4 * g4 + 3]};
+        if (half == 0) ws[RP] = m_run, ws[RP + 1] = l_run;
+        return;
+    }
     const float inv = 1.0f / l_run;
     float* out = p.out + ((size_t)(sp.row0 + row) * p.heads + head) * p.rank;
 #pragma unroll
@@ -235,7 +249,40 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(LatentAttent
         }
 }
 
+// a workgroup per item: out = sum_s e^(m_s - M) O_s / sum_s e^(m_s - M) l_s over the splits (a split that saw no key has l = 0 and m = -1e30: weight 0).
+// The splits' weights are formed once (one thread per split, through LDS); the sums over the splits run in split order.
+__global__ void __launch_bounds__(256) latent_attention_merge_kernel(const float* ws, float* out, uint32_t items, uint32_t splits, uint32_t rank, uint32_t rp) {
+    __shared__ float s_w[64];
+    __shared__ float s_inv;
+    const uint32_t item = blockIdx.x, tid = threadIdx.x;
+    const float* base = ws + (size_t)item * splits * (rp + 4);
+    if (tid < 64) {
+        const float m = tid < splits ? base[(size_t)tid * (rp + 4) + rp] : -1.0e30f;
+        const float M = wave_max(m);
+        const float w = fast_exp(m - M);
+        s_w[tid] = w;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        float L = 0.0f;
+        for (uint32_t s = 0; s < splits; ++s) L = fmaf(s_w[s], base[(size_t)s * (rp + 4) + rp + 1], L);
+        s_inv = 1.0f / L;
+    }
+    __syncthreads();
+    const float inv = s_inv;
+    for (uint32_t e = tid; e < rank; e += blockDim.x) {
+        float acc = 0.0f;
+        for (uint32_t s = 0; s < splits; ++s) acc = fmaf(s_w[s], base[(size_t)s * (rp + 4) + e], acc);
+        out[(size_t)item * rank + e] = acc * inv;
+    }
+}
+
 } // namespace
+
+size_t latent_attention_split_ws_bytes(uint32_t rows, uint32_t heads, uint32_t rank, uint32_t splits) {
+    const uint32_t rp = rank <= 128 ? 128 : 256;
+    return (size_t)rows * heads * splits * (rp + 4) * 4;
+}
 
 bool latent_attention_tiled_supported(const LatentAttentionParams& p) {
     return p.cache_bf16 && p.rank % 8 == 0 && p.rank <= 256 && p.nseq > 0 && p.tiles > 0 && (uintptr_t)p.qlat % 16 == 0 && (uintptr_t)p.out % 16 == 0;
@@ -255,15 +302,30 @@ uzu_status latent_attention(hipStream_t s, const LatentAttentionParams& p) {
     UZU_UNSUPPORTED(p.rank > kLatentMaxRank, "latent_attention: latent rank %u above %u", p.rank, kLatentMaxRank);
     UZU_UNSUPPORTED(p.form == 2 && !latent_attention_tiled_supported(p), "latent_attention: the tiled form takes a bf16 cache, rank %% 8 == 0, rank <= 256");
     if (p.form != 1 && latent_attention_tiled_supported(p)) {
-        static LdsLimit lim4, lim8;
-        if (p.rank <= 128) {
-            const size_t lds = 32 * (128 * 2 + 16) + 128 * 80;
-            raise_lds_limit(lim4, (const void*)latent_attention_mfma_kernel<4>, lds);
-            return launch_check([&] { hipLaunchKernelGGL(latent_attention_mfma_kernel<4>, dim3(p.tiles), dim3(256), lds, s, p); }, "latent_attention_mfma");
+        static LdsLimit lim4, lim8, lim4s, lim8s;
+        const uint32_t rp = p.rank <= 128 ? 128 : 256;
+        const size_t lds = 32 * (rp * 2 + 16) + rp * 80;
+        // few item tiles over many keys (decode steps): the key blocks of a tile are spread over `splits` workgroups and merged by a second launch
+        const uint32_t splits = (p.split_ws && p.splits > 1 && p.splits <= 64 && latent_attention_split_ws_bytes(p.rows, p.heads, p.rank, p.splits) <= p.split_ws_bytes) ? p.splits : 1;
+        if (splits > 1) {
+            const dim3 grid(p.tiles, splits);
+            if (rp == 128) {
+                raise_lds_limit(lim4s, (const void*)latent_attention_mfma_kernel<4, true>, lds);
+                UZU_PROPAGATE(launch_check([&] { hipLaunchKernelGGL((latent_attention_mfma_kernel<4, true>), grid, dim3(256), lds, s, p); }, "latent_attention_mfma_split"));
+            } else {
+                raise_lds_limit(lim8s, (const void*)latent_attention_mfma_kernel<8, true>, lds);
+                UZU_PROPAGATE(launch_check([&] { hipLaunchKernelGGL((latent_attention_mfma_kernel<8, true>), grid, dim3(256), lds, s, p); }, "latent_attention_mfma_split"));
+            }
+            const uint32_t items = p.rows * p.heads;
+            return launch_check([&] { hipLaunchKernelGGL(latent_attention_merge_kernel, dim3(items), dim3(256), 0, s, p.split_ws, p.out, items, splits, p.rank, rp); },
+                                "latent_attention_merge");
         }
-        const size_t lds = 32 * (256 * 2 + 16) + 256 * 80;
-        raise_lds_limit(lim8, (const void*)latent_attention_mfma_kernel<8>, lds);
-        return launch_check([&] { hipLaunchKernelGGL(latent_attention_mfma_kernel<8>, dim3(p.tiles), dim3(256), lds, s, p); }, "latent_attention_mfma");
+        if (rp == 128) {
+            raise_lds_limit(lim4, (const void*)latent_attention_mfma_kernel<4, false>, lds);
+            return launch_check([&] { hipLaunchKernelGGL((latent_attention_mfma_kernel<4, false>), dim3(p.tiles), dim3(256), lds, s, p); }, "latent_attention_mfma");
+        }
+        raise_lds_limit(lim8, (const void*)latent_attention_mfma_kernel<8, false>, lds);
+        return launch_check([&] { hipLaunchKernelGGL((latent_attention_mfma_kernel<8, false>), dim3(p.tiles), dim3(256), lds, s, p); }, "latent_attention_mfma");
     }
     const uint32_t items = p.rows * p.heads;
     const dim3 grid((items + 3) / 4), block(256);

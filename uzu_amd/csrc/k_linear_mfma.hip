@@ -22,7 +22,7 @@ constexpr int PITCH = 144;   // bytes per staged row: 64 bf16 + 16 bytes of pad
 
 __device__ __forceinline__ uint32_t pack_bf16(float a, float b) { return (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16); }
 
-template <int MB, int NB>
+template <int MB, int NB, bool GROUPED> // GROUPED: per-product row buckets (row_offsets) and gathered operand rows (row_map); the plain form carries neither
 __global__ void __launch_bounds__(256) linear_mfma_kernel(LinearF32Params p) {
     constexpr int BM = 64 * MB, BN = 64 * NB;
     constexpr int A_PASSES = BM / 16; // 16 threads cover a row's 64 k (one float4 each), 16 rows per pass
@@ -33,7 +33,13 @@ __global__ void __launch_bounds__(256) linear_mfma_kernel(LinearF32Params p) {
     const uint32_t z = blockIdx.z;
     const float* x = p.x + z * p.x_batch;
     const uint16_t* w = p.w + z * p.w_batch;
-    const uint32_t m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    uint32_t r_lo = 0, r_hi = p.rows;
+    if (GROUPED) { // a grouped launch: this product's bucket of rows (workgroup-uniform: the exit comes before any barrier)
+        r_lo = p.row_offsets[z], r_hi = p.row_offsets[z + 1];
+        x = p.x;
+    }
+    const uint32_t m0 = r_lo + blockIdx.y * BM, n0 = blockIdx.x * BN;
+    if (m0 >= r_hi) return;
 
     f32x16_t acc[MB][NB];
 #pragma unroll
@@ -51,8 +57,9 @@ __global__ void __launch_bounds__(256) linear_mfma_kernel(LinearF32Params p) {
 #pragma unroll
         for (int i = 0; i < A_PASSES; ++i) {
             const uint32_t r = m0 + a_row + i * 16, kk = k0 + a_k;
-            const bool ok = r < p.rows && kk < p.k;
-            const float* src = x + (size_t)(ok ? r : 0) * p.ldx + (ok ? kk : 0);
+            const bool ok = r < r_hi && kk < p.k;
+            const uint32_t sr = ok ? ((GROUPED && p.row_map) ? p.row_map[r] : r) : 0;
+            const float* src = x + (size_t)sr * p.ldx + (ok ? kk : 0);
             const f32x4_v v = *(const f32x4_v*)src;
             a_reg[i] = ok ? v : f32x4_v{0.f, 0.f, 0.f, 0.f};
         }
@@ -101,7 +108,7 @@ __global__ void __launch_bounds__(256) linear_mfma_kernel(LinearF32Params p) {
         }
     }
 
-    float* y = p.y + z * p.y_batch;
+    float* y = GROUPED ? p.y : p.y + z * p.y_batch;
 #pragma unroll
     for (int j = 0; j < NB; ++j) {
         const uint32_t n = n0 + (wn * NB + j) * 32 + l32;
@@ -112,7 +119,7 @@ __global__ void __launch_bounds__(256) linear_mfma_kernel(LinearF32Params p) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const uint32_t row = m0 + (wm * MB + i) * 32 + (r & 3) + 8 * (r >> 2) + 4 * half;
-                if (row >= p.rows) continue;
+                if (row >= r_hi) continue;
                 float v = acc[i][j][r] + bias;
                 if (p.act == 1) {
                     const float t = fmaxf(v, 0.0f);
@@ -128,29 +135,35 @@ __global__ void __launch_bounds__(256) linear_mfma_kernel(LinearF32Params p) {
 } // namespace
 
 bool linear_mfma_supported(const LinearF32Params& p) {
-    if (!p.bf16_products || p.rows < 32 || p.k % 8 || p.ldx % 4 || p.x_batch % 4 || p.w_batch % 8) return false;
+    if (!p.bf16_products || (p.rows < 32 && !p.row_offsets) || p.k % 8 || p.ldx % 4 || p.x_batch % 4 || p.w_batch % 8) return false;
     if ((uintptr_t)p.x % 16 || (uintptr_t)p.w % 16) return false;
     return true;
 }
 
 uzu_status linear_mfma(hipStream_t s, const LinearF32Params& p) {
     UZU_REQUIRE(linear_mfma_supported(p), "linear_mfma: shape / alignment not covered");
+    UZU_REQUIRE(p.row_offsets || !p.row_map, "linear_mfma: gathered rows only in the grouped form");
     // tile choice: the widest tile that still fills the chip; narrow outputs (the per-head products) take the narrow tiles
+    if (p.row_offsets) { // grouped: every product may need the whole row range, the workgroups beyond a bucket leave at once
+        const dim3 grid((p.n + 127) / 128, (p.rows + 127) / 128 + 1, p.batch);
+        UZU_REQUIRE(grid.y <= 65535 && grid.z <= 65535 && !p.residual, "linear_mfma: grouped grid too large");
+        return launch_check([&] { hipLaunchKernelGGL((linear_mfma_kernel<2, 2, true>), grid, dim3(256), 0, s, p); }, "linear_mfma_grouped");
+    }
     const bool small_m = p.rows <= 64, small_n = p.n <= 64;
     auto tiles = [&](uint32_t bm, uint32_t bn) { return (size_t)((p.rows + bm - 1) / bm) * ((p.n + bn - 1) / bn) * p.batch; };
     if (!small_m && !small_n && tiles(128, 128) >= 256) {
         const dim3 grid((p.n + 127) / 128, (p.rows + 127) / 128, p.batch);
         UZU_REQUIRE(grid.y <= 65535 && grid.z <= 65535, "linear_mfma: grid too large");
-        return launch_check([&] { hipLaunchKernelGGL((linear_mfma_kernel<2, 2>), grid, dim3(256), 0, s, p); }, "linear_mfma<2,2>");
+        return launch_check([&] { hipLaunchKernelGGL((linear_mfma_kernel<2, 2, false>), grid, dim3(256), 0, s, p); }, "linear_mfma<2,2>");
     }
     if (!small_m && (small_n || tiles(128, 64) >= 256)) {
         const dim3 grid((p.n + 63) / 64, (p.rows + 127) / 128, p.batch);
         UZU_REQUIRE(grid.y <= 65535 && grid.z <= 65535, "linear_mfma: grid too large");
-        return launch_check([&] { hipLaunchKernelGGL((linear_mfma_kernel<2, 1>), grid, dim3(256), 0, s, p); }, "linear_mfma<2,1>");
+        return launch_check([&] { hipLaunchKernelGGL((linear_mfma_kernel<2, 1, false>), grid, dim3(256), 0, s, p); }, "linear_mfma<2,1>");
     }
     const dim3 grid((p.n + 63) / 64, (p.rows + 63) / 64, p.batch);
     UZU_REQUIRE(grid.y <= 65535 && grid.z <= 65535, "linear_mfma: grid too large");
-    return launch_check([&] { hipLaunchKernelGGL((linear_mfma_kernel<1, 1>), grid, dim3(256), 0, s, p); }, "linear_mfma<1,1>");
+    return launch_check([&] { hipLaunchKernelGGL((linear_mfma_kernel<1, 1, false>), grid, dim3(256), 0, s, p); }, "linear_mfma<1,1>");
 }
 
 } // namespace k

@@ -13,6 +13,26 @@ namespace {
 
 __device__ __forceinline__ float opnd(float v, uint32_t bf16_products) { return bf16_products ? round_bf16(v) : v; }
 
+// this lane's share of <x, w> over n elements (x f32 in LDS or global, w bf16 in global): 16-byte weight loads where the row allows them (n % 8 == 0 and
+// the row 16-byte aligned), element loads otherwise; the caller sums over the wave
+__device__ __forceinline__ float lane_dot(const float* x, const uint16_t* w, uint32_t n, uint32_t lane) {
+    float acc = 0.0f;
+    if ((n & 7) == 0 && ((uintptr_t)w & 15) == 0) {
+        for (uint32_t i0 = lane * 8; i0 < n; i0 += 512) {
+            const uint4 wv = *(const uint4*)(w + i0);
+            const uint32_t ww[4] = {wv.x, wv.y, wv.z, wv.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                acc = fmaf(x[i0 + 2 * j], bits_to_f32(ww[j] << 16), acc);
+                acc = fmaf(x[i0 + 2 * j + 1], bits_to_f32(ww[j] & 0xFFFF0000u), acc);
+            }
+        }
+    } else {
+        for (uint32_t i = lane; i < n; i += 64) acc = fmaf(x[i], bf16_to_f32(w[i]), acc);
+    }
+    return acc;
+}
+
 __global__ void __launch_bounds__(256) embed_rows_f32_kernel(const uint32_t* tokens, const uint16_t* table, float* out, uint32_t vocab, uint32_t d) {
     const uint32_t r = blockIdx.x;
     uint32_t t = tokens[r];
@@ -27,8 +47,9 @@ __global__ void __launch_bounds__(256) dyn_tanh_kernel(DynTanhParams p) {
     const uint32_t src = p.row_index ? p.row_index[r] : r;
     const float* x = p.x + (size_t)src * p.d;
     float* out = p.out + (size_t)r * p.d;
+    const uint32_t i0 = blockIdx.y * blockDim.x + threadIdx.x, step = gridDim.y * blockDim.x; // a row is spread over grid.y workgroups: one round of loads per thread
     if (!p.shift) {
-        for (uint32_t i = threadIdx.x; i < p.d; i += blockDim.x) out[i] = fmaf(tanhf(p.alpha * x[i]), p.scales[i], p.biases ? p.biases[i] : 0.0f);
+        for (uint32_t i = i0; i < p.d; i += step) out[i] = fmaf(tanhf(p.alpha * x[i]), p.scales[i], p.biases ? p.biases[i] : 0.0f);
         return;
     }
     const uint32_t q = p.row_seq[r];
@@ -36,7 +57,7 @@ __global__ void __launch_bounds__(256) dyn_tanh_kernel(DynTanhParams p) {
     const bool first = r == sp.row0;
     float* prev = p.prev[q];
     const float* xl = p.x + (size_t)(sp.row0 + sp.count - 1) * p.d; // the sequence's last row of the pass
-    for (uint32_t i = threadIdx.x; i < p.d; i += blockDim.x) {
+    for (uint32_t i = i0; i < p.d; i += step) {
         const float w = p.scales[i], b = p.biases ? p.biases[i] : 0.0f;
         const float h = fmaf(tanhf(p.alpha * x[i]), w, b);
         float hp;
@@ -188,10 +209,7 @@ __global__ void __launch_bounds__(64) moe_route_scores_kernel(const float* x, co
 #pragma unroll
     for (int j = 0; j < 8; ++j) z[j] = -INFINITY;
     for (uint32_t e = 0; e < outputs; ++e) {
-        const uint16_t* w = router + (size_t)e * d;
-        float acc = 0.0f;
-        for (uint32_t i = lane; i < d; i += 64) acc = fmaf(xr[i], bf16_to_f32(w[i]), acc);
-        acc = wave_sum(acc);
+        float acc = wave_sum(lane_dot(xr, router + (size_t)e * d, d, lane));
         if ((e & 63) == lane) {
 #pragma unroll
             for (int j = 0; j < 8; ++j)
@@ -262,13 +280,7 @@ __global__ void __launch_bounds__(256) moe_experts_gate_up_kernel(const float* x
     for (uint32_t f = blockIdx.y * nw + wave; f < ff; f += gridDim.y * nw) {
         const uint16_t* wu = base + (size_t)f * d;
         const uint16_t* wg = base + (size_t)(ff + f) * d;
-        float au = 0.0f, ag = 0.0f;
-        for (uint32_t i = lane; i < d; i += 64) {
-            const float xv = s_x[i];
-            au = fmaf(xv, bf16_to_f32(wu[i]), au);
-            ag = fmaf(xv, bf16_to_f32(wg[i]), ag);
-        }
-        au = wave_sum(au), ag = wave_sum(ag);
+        const float au = wave_sum(lane_dot(s_x, wu, d, lane)), ag = wave_sum(lane_dot(s_x, wg, d, lane));
         if (lane == 0) hidden[(size_t)slot * ff + f] = ag / (1.0f + expf(-ag)) * au;
     }
 }
@@ -294,17 +306,100 @@ __global__ void __launch_bounds__(256) moe_experts_down_kernel(const float* hidd
                 total = fmaf(wt, x[(size_t)r * d + n], total);
                 continue;
             }
-            const uint16_t* w = w2 + ((size_t)e * d + n) * ff;
-            float acc = 0.0f;
-            for (uint32_t i = lane; i < ff; i += 64) acc = fmaf(s_h[j * ff + i], bf16_to_f32(w[i]), acc);
-            acc = wave_sum(acc);
+            const float acc = wave_sum(lane_dot(s_h + j * ff, w2 + ((size_t)e * d + n) * ff, ff, lane));
             total = fmaf(wt, acc, total);
         }
         if (lane == 0) y[(size_t)r * d + n] = total;
     }
 }
 
+// ---- bucketing of the (row, slot) pairs by expert for the grouped matrix-core form
+__global__ void __launch_bounds__(1024) moe_bucket_kernel(const int32_t* ids, uint32_t slots, uint32_t routed, uint32_t* offsets, uint32_t* cursor) {
+    extern __shared__ uint32_t s_hist[];
+    for (uint32_t e = threadIdx.x; e < routed; e += blockDim.x) s_hist[e] = 0;
+    __syncthreads();
+    for (uint32_t i = threadIdx.x; i < slots; i += blockDim.x) {
+        const int32_t e = ids[i];
+        if (e >= 0 && (uint32_t)e < routed) atomicAdd(&s_hist[e], 1u);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t run = 0;
+        for (uint32_t e = 0; e < routed; ++e) {
+            offsets[e] = run, cursor[e] = 0;
+            run += s_hist[e];
+        }
+        offsets[routed] = run;
+    }
+}
+// a pair's place inside its expert's bucket: the order of arrival (any order gives the same numbers: a row's product does not depend on its place in a tile)
+__global__ void __launch_bounds__(256) moe_scatter_kernel(const int32_t* ids, uint32_t slots, uint32_t routed, uint32_t top, const uint32_t* offsets, uint32_t* cursor, uint32_t* perm,
+                                                         uint32_t* slot_pos) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= slots) return;
+    const int32_t e = ids[i];
+    if (e < 0 || (uint32_t)e >= routed) {
+        slot_pos[i] = 0xFFFFFFFFu;
+        return;
+    }
+    const uint32_t pos = offsets[e] + atomicAdd(&cursor[e], 1u);
+    perm[pos] = i / top;
+    slot_pos[i] = pos;
+}
+__global__ void __launch_bounds__(256) moe_act_mul_kernel(const float* y1, float* hidden, const uint32_t* offsets, uint32_t routed, uint32_t ff) {
+    const uint32_t pos = blockIdx.x;
+    if (pos >= offsets[routed]) return;
+    const float* src = y1 + (size_t)pos * 2 * ff;
+    for (uint32_t f = threadIdx.x; f < ff; f += blockDim.x) {
+        const float g = src[ff + f];
+        hidden[(size_t)pos * ff + f] = g / (1.0f + expf(-g)) * src[f];
+    }
+}
+__global__ void __launch_bounds__(256) moe_combine_kernel(const float* y2, const float* x, const int32_t* ids, const float* weights, const uint32_t* slot_pos, const float* residual,
+                                                         float* y, uint32_t d, uint32_t routed, uint32_t top) {
+    const uint32_t r = blockIdx.x;
+    for (uint32_t n = threadIdx.x; n < d; n += blockDim.x) {
+        float total = residual ? residual[(size_t)r * d + n] : 0.0f;
+        for (uint32_t j = 0; j < top; ++j) {
+            const int32_t e = ids[(size_t)r * top + j];
+            if (e < 0) continue;
+            const float src = (uint32_t)e >= routed ? x[(size_t)r * d + n] : y2[(size_t)slot_pos[(size_t)r * top + j] * d + n];
+            total = fmaf(weights[(size_t)r * top + j], src, total);
+        }
+        y[(size_t)r * d + n] = total;
+    }
+}
+
 } // namespace
+
+bool moe_experts_grouped_supported(const MoeGroupedParams& p) {
+    if (!p.routed || p.rows < 64 || p.routed > 8192 || !p.y1 || !p.y2 || !p.hidden || !p.perm) return false;
+    LinearF32Params q{};
+    q.x = p.x, q.w = p.w13, q.y = p.y1, q.rows = p.rows * p.top, q.n = 2 * p.ff, q.k = p.d, q.ldx = p.d, q.ldy = 2 * p.ff, q.batch = p.routed, q.w_batch = (size_t)2 * p.ff * p.d;
+    q.bf16_products = 1, q.row_offsets = p.offsets, q.row_map = p.perm;
+    LinearF32Params r = q;
+    r.x = p.hidden, r.w = p.w2, r.y = p.y2, r.n = p.d, r.k = p.ff, r.ldx = p.ff, r.ldy = p.d, r.w_batch = (size_t)p.d * p.ff, r.row_map = nullptr;
+    return linear_mfma_supported(q) && linear_mfma_supported(r);
+}
+
+uzu_status moe_experts_grouped(hipStream_t s, const MoeGroupedParams& p) {
+    UZU_REQUIRE(moe_experts_grouped_supported(p), "moe_experts_grouped: shape not covered");
+    const uint32_t slots = p.rows * p.top;
+    UZU_PROPAGATE(launch_check([&] { hipLaunchKernelGGL(moe_bucket_kernel, dim3(1), dim3(1024), (size_t)p.routed * 4, s, p.ids, slots, p.routed, p.offsets, p.cursor); }, "moe_bucket"));
+    UZU_PROPAGATE(launch_check([&] { hipLaunchKernelGGL(moe_scatter_kernel, dim3((slots + 255) / 256), dim3(256), 0, s, p.ids, slots, p.routed, p.top, p.offsets, p.cursor, p.perm, p.slot_pos); },
+                               "moe_scatter"));
+    LinearF32Params q{};
+    q.x = p.x, q.w = p.w13, q.y = p.y1, q.rows = slots, q.n = 2 * p.ff, q.k = p.d, q.ldx = p.d, q.ldy = 2 * p.ff, q.batch = p.routed, q.w_batch = (size_t)2 * p.ff * p.d;
+    q.bf16_products = 1, q.row_offsets = p.offsets, q.row_map = p.perm;
+    UZU_PROPAGATE(linear_mfma(s, q));
+    UZU_PROPAGATE(launch_check([&] { hipLaunchKernelGGL(moe_act_mul_kernel, dim3(slots), dim3(256), 0, s, p.y1, p.hidden, p.offsets, p.routed, p.ff); }, "moe_act_mul"));
+    LinearF32Params r{};
+    r.x = p.hidden, r.w = p.w2, r.y = p.y2, r.rows = slots, r.n = p.d, r.k = p.ff, r.ldx = p.ff, r.ldy = p.d, r.batch = p.routed, r.w_batch = (size_t)p.d * p.ff;
+    r.bf16_products = 1, r.row_offsets = p.offsets;
+    UZU_PROPAGATE(linear_mfma(s, r));
+    return launch_check([&] { hipLaunchKernelGGL(moe_combine_kernel, dim3(p.rows), dim3(256), 0, s, p.y2, p.x, p.ids, p.weights, p.slot_pos, p.residual, p.y, p.d, p.routed, p.top); },
+                        "moe_combine");
+}
 
 uzu_status embed_rows_f32(hipStream_t s, const uint32_t* tokens, const uint16_t* table, float* out, uint32_t rows, uint32_t vocab, uint32_t d) {
     if (!rows) return UZU_OK;
@@ -316,7 +411,8 @@ uzu_status dyn_tanh_norm(hipStream_t s, const DynTanhParams& p) {
     UZU_REQUIRE(p.x && p.out && p.scales, "dyn_tanh_norm: null argument");
     UZU_REQUIRE(!p.shift || (p.spans && p.row_seq && p.prev && !p.row_index), "dyn_tanh_norm: the token shift needs the pass's spans, row map and state rows");
     UZU_REQUIRE(!p.shift || p.x != p.out, "dyn_tanh_norm: the token shift reads neighbouring rows: not in place");
-    return launch_check([&] { hipLaunchKernelGGL(dyn_tanh_kernel, dim3(p.rows), dim3(256), 0, s, p); }, "dyn_tanh_norm");
+    const uint32_t gy = p.rows >= 1024 ? 1 : (p.d + 255) / 256 < 64 ? (p.d + 255) / 256 : 64;
+    return launch_check([&] { hipLaunchKernelGGL(dyn_tanh_kernel, dim3(p.rows, gy), dim3(256), 0, s, p); }, "dyn_tanh_norm");
 }
 
 uzu_status depth_mix(hipStream_t s, const float* slots, size_t slot_stride, const float* w, uint32_t count, float* out, uint32_t rows, uint32_t d) {
@@ -332,6 +428,11 @@ uzu_status linear_f32(hipStream_t s, const LinearF32Params& p, const char** vari
     UZU_REQUIRE(p.x && p.w && p.y && p.k, "linear_f32: null argument");
     UZU_REQUIRE(!p.residual || p.batch == 1, "linear_f32: a residual only with one product per launch");
     UZU_REQUIRE(p.ldx >= p.k && p.ldy >= p.n && p.batch <= 65535, "linear_f32: row pitch below the row length");
+    if (p.row_offsets || p.row_map) { // the grouped / gathered form lives in the matrix-core kernel only
+        UZU_UNSUPPORTED(!linear_mfma_supported(p), "linear_f32: grouped / gathered rows need bf16 products and 8-aligned k");
+        if (variant) *variant = "linear_mfma_grouped";
+        return linear_mfma(s, p);
+    }
     if (p.rows <= 16) {
         const uint32_t vec = (p.k % 8 == 0 && p.ldx % 4 == 0 && p.x_batch % 4 == 0 && p.w_batch % 8 == 0 && (uintptr_t)p.x % 16 == 0 && (uintptr_t)p.w % 16 == 0) ? 1u : 0u;
         if (variant) *variant = "linear_rows";
@@ -363,7 +464,9 @@ uzu_status moe_experts_gate_up(hipStream_t s, const float* x, const int32_t* ids
                                uint32_t top, uint32_t bf16_products) {
     if (!rows || !routed) return UZU_OK;
     UZU_UNSUPPORTED((size_t)d * 4 > 64 * 1024, "moe_experts_gate_up: model_dim %u does not fit the workgroup's LDS row", d);
-    const uint32_t gy = ff >= 256 ? 4 : 1; // wide experts: several workgroups share a (row, slot)
+    // few (row, slot) pairs (decode): the hidden units of a pair are spread over more workgroups, so that the expert's rows stream through many CUs
+    const uint32_t want = (1024 + rows * top - 1) / (rows * top), most = (ff + 15) / 16;
+    const uint32_t gy = want < 1 ? 1 : (want > most ? most : want);
     return launch_check([&] { hipLaunchKernelGGL(moe_experts_gate_up_kernel, dim3(rows * top, gy), dim3(256), (size_t)d * 4, s, x, ids, w13, hidden, d, ff, routed, top, bf16_products); },
                         "moe_experts_gate_up");
 }
@@ -372,7 +475,8 @@ uzu_status moe_experts_down_combine(hipStream_t s, const float* hidden, const fl
                                     float* y, uint32_t rows, uint32_t d, uint32_t ff, uint32_t routed, uint32_t top, uint32_t bf16_products) {
     if (!rows) return UZU_OK;
     UZU_UNSUPPORTED((size_t)top * ff * 4 > 64 * 1024, "moe_experts_down_combine: %u slots x %u hidden units do not fit the workgroup's LDS", top, ff);
-    const uint32_t gy = d >= 1024 ? 4 : 1;
+    const uint32_t want = (1024 + rows - 1) / rows, most = (d + 15) / 16;
+    const uint32_t gy = want < 1 ? 1 : (want > most ? most : want);
     return launch_check([&] { hipLaunchKernelGGL(moe_experts_down_kernel, dim3(rows, gy), dim3(256), (size_t)top * ff * 4, s, hidden, x, ids, weights, w2, residual, y, d, ff, routed, top,
                                                   bf16_products); }, "moe_experts_down_combine");
 }

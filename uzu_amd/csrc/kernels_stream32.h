@@ -60,6 +60,11 @@ struct LinearF32Params {
     size_t x_batch, w_batch, y_batch; // element strides
     uint32_t act;
     uint32_t bf16_products;
+    // Grouped form (matrix-core kernel only; the experts of a mixture, each with its own bucket of rows): product z covers rows row_offsets[z] ..
+    // row_offsets[z + 1] - 1 of X and Y (device array [batch + 1]; x_batch / y_batch unused, `rows` = an upper bound of the total for the grid).
+    const uint32_t* row_offsets;
+    // row r of X is x[row_map[r]] (device array, or null): a gather folded into the operand load
+    const uint32_t* row_map;
 };
 uzu_status linear_f32(hipStream_t s, const LinearF32Params& p, const char** variant = nullptr);
 // the matrix-core form (k_linear_mfma.hip): bf16 products only; false = shape / mode not covered, nothing launched
@@ -77,6 +82,23 @@ uzu_status moe_experts_gate_up(hipStream_t s, const float* x, const int32_t* ids
 // y[r, :] = residual[r, :] + sum_j weights[r, j] * (ids[r, j] < routed ? down_e hidden[r * top + j] : x[r, :])   in slot order; w2 bf16 [routed][d][ff]; y may alias residual
 uzu_status moe_experts_down_combine(hipStream_t s, const float* hidden, const float* x, const int32_t* ids, const float* weights, const uint16_t* w2, const float* residual,
                                     float* y, uint32_t rows, uint32_t d, uint32_t ff, uint32_t routed, uint32_t top, uint32_t bf16_products);
+
+// The same block for prefill-sized row counts with bf16 products: the (row, slot) pairs are bucketed by expert (counts -> offsets -> positions), every expert runs
+// its bucket through the matrix-core linear as one grouped launch (gate | up, then down), and the rows are combined in slot order.  Workspaces: y1
+// [rows * top][2 ff], hidden [rows * top][ff], y2 [rows * top][d] f32; perm / slot_pos [rows * top], offsets [routed + 1], cursor [routed] u32.
+struct MoeGroupedParams {
+    const float* x;
+    const int32_t* ids;
+    const float* weights;
+    const uint16_t *w13, *w2;
+    const float* residual;
+    float* y;
+    float *y1, *hidden, *y2;
+    uint32_t *perm, *slot_pos, *offsets, *cursor;
+    uint32_t rows, d, ff, routed, top;
+};
+bool moe_experts_grouped_supported(const MoeGroupedParams& p);
+uzu_status moe_experts_grouped(hipStream_t s, const MoeGroupedParams& p);
 
 // RMS norm of the latent rows (x / sqrt(mean(x^2) + eps) * scales) and append to the sequences' caches: row r goes to cache[seq(r)] + (position of r) * rank,
 // stored as bf16 (cache_bf16) or f32.
@@ -99,7 +121,13 @@ struct LatentAttentionParams {
     uint32_t form; // 0: chosen by shape; 1: the simple form (a wave per row and head, keys one after the other); 2: the tiled form
     uint32_t nseq;  // entries of `spans`
     uint32_t tiles; // sum over the sequences of ceil(count * heads / 128): the tiled form's workgroups (the caller knows the counts)
+    // tiled form, few rows over many keys (decode): `splits` > 1 workgroups share the key blocks of an item tile, partial sums go through split_ws
+    // (latent_attention_split_ws_bytes(rows, heads, rank, splits) bytes) and a merge launch.  0 / null: one workgroup walks all keys of its tile.
+    uint32_t splits;
+    float* split_ws;
+    size_t split_ws_bytes;
 };
+size_t latent_attention_split_ws_bytes(uint32_t rows, uint32_t heads, uint32_t rank, uint32_t splits);
 bool latent_attention_tiled_supported(const LatentAttentionParams& p);
 uzu_status latent_attention(hipStream_t s, const LatentAttentionParams& p);
 constexpr uint32_t kLatentMaxRank = 1024;

@@ -209,3 +209,21 @@ def test_refusals(models, hip_ctx):
     with pytest.raises(UzuHipError):
         m.step_batch([st], [[1] * 600], [[]])                # beyond max_context_length
     st.close()
+
+
+def test_generate_loop_of_the_text_front_end_on_token_ids(hip_ctx, tmp_path):
+    """LanguageModel.generate (the engine's generate loop: prefill, chained decode in chunks, stop tokens) on a directory without tokenizer.json"""
+    from uzu_amd.language_model import LanguageModel, TokenizerError
+    cfg = cfg_a()
+    W = O.weights(cfg, 31)
+    O.write_model_dir(str(tmp_path / "g"), cfg, W)
+    W64 = {k: v.astype(np.float64) for k, v in W.items()}
+    with pytest.raises(TokenizerError):
+        LanguageModel(hip_ctx, str(tmp_path / "g"), max_context_length=128)
+    lm = LanguageModel(hip_ctx, str(tmp_path / "g"), max_context_length=128, flags=MODEL_FULL_F32, tokenizer_required=False)
+    p = prompt(cfg, 12, 3)
+    res = lm.generate(p, max_tokens=11, chunk=4)
+    assert res.token_ids == O.greedy(cfg, W64, p, 11) and res.prompt_tokens == 12 and res.stopped_on is None
+    with pytest.raises(TokenizerError):
+        lm.generate("text", max_tokens=2)
+    lm.close()

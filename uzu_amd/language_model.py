@@ -77,12 +77,17 @@ def read_generation_config(model_dir: str) -> GenerationConfig:
 class LanguageModel:
     """config.json + model.safetensors + tokenizer.json -> text in, text out on the HIP engine."""
 
-    def __init__(self, ctx: Context, model_dir: str, max_context_length: Optional[int] = None, flags: int = MODEL_DEFAULT):
+    def __init__(self, ctx: Context, model_dir: str, max_context_length: Optional[int] = None, flags: int = MODEL_DEFAULT, tokenizer_required: bool = True):
+        """The model class follows config.json (uzu_amd.loader.load_model_dir: the reference's schema, or a design named by `architecture`).
+        `tokenizer_required=False`: a directory without tokenizer.json serves token ids only (generate() then takes and returns ids; text raises)."""
         self.ctx = ctx
-        self.tokenizer = load_tokenizer(model_dir)
+        if tokenizer_required or os.path.exists(os.path.join(model_dir, "tokenizer.json")):
+            self.tokenizer = load_tokenizer(model_dir)
+        else:
+            self.tokenizer = None
         self.generation_config = read_generation_config(model_dir)
         self.bundle = loader.load_model_dir(model_dir, max_context_length=max_context_length)
-        vocab = self.tokenizer.get_vocab_size(with_added_tokens=True)
+        vocab = self.tokenizer.get_vocab_size(with_added_tokens=True) if self.tokenizer is not None else 0
         if vocab > self.bundle.vocab_size:
             raise TokenizerError(f"tokenizer.json has {vocab} tokens, the model's embedding {self.bundle.vocab_size} rows")
         self.model = HipModel(ctx, self.bundle, flags)
@@ -92,9 +97,13 @@ class LanguageModel:
 
     # ---- text <-> ids
     def encode(self, text: str, add_special_tokens: bool = True) -> List[int]:
+        if self.tokenizer is None:
+            raise TokenizerError("this model directory has no tokenizer.json: pass token ids")
         return list(self.tokenizer.encode(text, add_special_tokens=add_special_tokens).ids)
 
     def decode(self, ids: Sequence[int], skip_special_tokens: bool = True) -> str:
+        if self.tokenizer is None:
+            return ""
         return self.tokenizer.decode([int(t) for t in ids], skip_special_tokens=skip_special_tokens)
 
     # ---- generation

@@ -334,7 +334,8 @@ uzu_status latent_attention(hipStream_t s, const LatentAttentionParams& p) {
     if (nt <= 2) return launch_check([&] { hipLaunchKernelGGL(latent_attention_rows_kernel<2>, grid, block, 0, s, p); }, "latent_attention");
     if (nt <= 4) return launch_check([&] { hipLaunchKernelGGL(latent_attention_rows_kernel<4>, grid, block, 0, s, p); }, "latent_attention");
     if (nt <= 8) return launch_check([&] { hipLaunchKernelGGL(latent_attention_rows_kernel<8>, grid, block, 0, s, p); }, "latent_attention");
-    return launch_check([&] { hipLaunchKernelGGL(latent_attention_rows_kernel<16>, grid, block, 0, s, p); }, "latent_attention");
+    if (nt <= 16) return launch_check([&] { hipLaunchKernelGGL(latent_attention_rows_kernel<16>, grid, block, 0, s, p); }, "latent_attention");
+    return launch_check([&] { hipLaunchKernelGGL(latent_attention_rows_kernel<32>, grid, block, 0, s, p); }, "latent_attention");
 }
 
 } // namespace k

@@ -15,8 +15,12 @@ __device__ __forceinline__ float opnd(float v, uint32_t bf16_products) { return 
 
 // this lane's share of <x, w> over n elements (x f32 in LDS or global, w bf16 in global): 16-byte weight loads where the row allows them (n % 8 == 0 and
 // the row 16-byte aligned), element loads otherwise; the caller sums over the wave
-__device__ __forceinline__ float lane_dot(const float* x, const uint16_t* w, uint32_t n, uint32_t lane) {
+__device__ __forceinline__ float lane_dot(const float* x, const uint16_t* w, uint32_t n, uint32_t lane, uint32_t round_x = 0) {
     float acc = 0.0f;
+    if (round_x) { // operand rows that were not rounded when they were staged (read straight from global memory)
+        for (uint32_t i = lane; i < n; i += 64) acc = fmaf(round_bf16(x[i]), bf16_to_f32(w[i]), acc);
+        return acc;
+    }
     if ((n & 7) == 0 && ((uintptr_t)w & 15) == 0) {
         for (uint32_t i0 = lane * 8; i0 < n; i0 += 512) {
             const uint4 wv = *(const uint4*)(w + i0);
@@ -287,14 +291,17 @@ __global__ void __launch_bounds__(256) moe_experts_gate_up_kernel(const float* x
 
 // a workgroup per (row, block of outputs): the row's hidden rows into LDS, then a wave per output; the slots are added in slot order
 __global__ void __launch_bounds__(256) moe_experts_down_kernel(const float* hidden, const float* x, const int32_t* ids, const float* weights, const uint16_t* w2,
-                                                               const float* residual, float* y, uint32_t d, uint32_t ff, uint32_t routed, uint32_t top, uint32_t bf16_products) {
-    extern __shared__ float s_h[]; // [top][ff]
+                                                               const float* residual, float* y, uint32_t d, uint32_t ff, uint32_t routed, uint32_t top, uint32_t bf16_products,
+                                                               uint32_t staged) {
+    extern __shared__ float s_h[]; // [top][ff] (staged; hidden rows too wide for LDS are read from global memory)
     const uint32_t r = blockIdx.x;
-    for (uint32_t i = threadIdx.x; i < top * ff; i += blockDim.x) {
-        const int32_t e = ids[(size_t)r * top + i / ff];
-        s_h[i] = (e >= 0 && (uint32_t)e < routed) ? opnd(hidden[(size_t)r * top * ff + i], bf16_products) : 0.0f;
+    if (staged) {
+        for (uint32_t i = threadIdx.x; i < top * ff; i += blockDim.x) {
+            const int32_t e = ids[(size_t)r * top + i / ff];
+            s_h[i] = (e >= 0 && (uint32_t)e < routed) ? opnd(hidden[(size_t)r * top * ff + i], bf16_products) : 0.0f;
+        }
+        __syncthreads();
     }
-    __syncthreads();
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
     for (uint32_t n = blockIdx.y * nw + wave; n < d; n += gridDim.y * nw) {
         float total = residual ? residual[(size_t)r * d + n] : 0.0f;
@@ -306,7 +313,8 @@ __global__ void __launch_bounds__(256) moe_experts_down_kernel(const float* hidd
                 total = fmaf(wt, x[(size_t)r * d + n], total);
                 continue;
             }
-            const float acc = wave_sum(lane_dot(s_h + j * ff, w2 + ((size_t)e * d + n) * ff, ff, lane));
+            const float* hrow = staged ? s_h + j * ff : hidden + ((size_t)r * top + j) * ff;
+            const float acc = wave_sum(lane_dot(hrow, w2 + ((size_t)e * d + n) * ff, ff, lane, staged ? 0u : bf16_products));
             total = fmaf(wt, acc, total);
         }
         if (lane == 0) y[(size_t)r * d + n] = total;
@@ -463,7 +471,7 @@ uzu_status moe_route_scores(hipStream_t s, const float* x, const uint16_t* route
 uzu_status moe_experts_gate_up(hipStream_t s, const float* x, const int32_t* ids, const uint16_t* w13, float* hidden, uint32_t rows, uint32_t d, uint32_t ff, uint32_t routed,
                                uint32_t top, uint32_t bf16_products) {
     if (!rows || !routed) return UZU_OK;
-    UZU_UNSUPPORTED((size_t)d * 4 > 64 * 1024, "moe_experts_gate_up: model_dim %u does not fit the workgroup's LDS row", d);
+    UZU_UNSUPPORTED((size_t)d * 4 > 48 * 1024, "moe_experts_gate_up: model_dim %u does not fit the workgroup's LDS row", d);
     // few (row, slot) pairs (decode): the hidden units of a pair are spread over more workgroups, so that the expert's rows stream through many CUs
     const uint32_t want = (1024 + rows * top - 1) / (rows * top), most = (ff + 15) / 16;
     const uint32_t gy = want < 1 ? 1 : (want > most ? most : want);
@@ -474,11 +482,11 @@ uzu_status moe_experts_gate_up(hipStream_t s, const float* x, const int32_t* ids
 uzu_status moe_experts_down_combine(hipStream_t s, const float* hidden, const float* x, const int32_t* ids, const float* weights, const uint16_t* w2, const float* residual,
                                     float* y, uint32_t rows, uint32_t d, uint32_t ff, uint32_t routed, uint32_t top, uint32_t bf16_products) {
     if (!rows) return UZU_OK;
-    UZU_UNSUPPORTED((size_t)top * ff * 4 > 64 * 1024, "moe_experts_down_combine: %u slots x %u hidden units do not fit the workgroup's LDS", top, ff);
+    const uint32_t staged = (size_t)top * ff * 4 <= 48 * 1024 ? 1u : 0u;
     const uint32_t want = (1024 + rows - 1) / rows, most = (d + 15) / 16;
     const uint32_t gy = want < 1 ? 1 : (want > most ? most : want);
-    return launch_check([&] { hipLaunchKernelGGL(moe_experts_down_kernel, dim3(rows, gy), dim3(256), (size_t)top * ff * 4, s, hidden, x, ids, weights, w2, residual, y, d, ff, routed, top,
-                                                  bf16_products); }, "moe_experts_down_combine");
+    return launch_check([&] { hipLaunchKernelGGL(moe_experts_down_kernel, dim3(rows, gy), dim3(256), staged ? (size_t)top * ff * 4 : 0, s, hidden, x, ids, weights, w2, residual, y, d, ff, routed, top,
+                                                  bf16_products, staged); }, "moe_experts_down_combine");
 }
 
 } // namespace k

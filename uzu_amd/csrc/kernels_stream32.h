@@ -130,7 +130,7 @@ struct LatentAttentionParams {
 size_t latent_attention_split_ws_bytes(uint32_t rows, uint32_t heads, uint32_t rank, uint32_t splits);
 bool latent_attention_tiled_supported(const LatentAttentionParams& p);
 uzu_status latent_attention(hipStream_t s, const LatentAttentionParams& p);
-constexpr uint32_t kLatentMaxRank = 1024;
+constexpr uint32_t kLatentMaxRank = 2048;
 
 } // namespace k
 } // namespace uzu

@@ -227,3 +227,22 @@ def test_generate_loop_of_the_text_front_end_on_token_ids(hip_ctx, tmp_path):
     with pytest.raises(TokenizerError):
         lm.generate("text", max_tokens=2)
     lm.close()
+
+
+def test_pool_generates_several_prompts_together(models):
+    """uzu_amd.serving.SequencePool: prompts of unequal length prefilled in one batch and decoded together, requests leaving as they finish (one by a stop
+    token), their states reused by a second round -- against each prompt generated alone by the oracle"""
+    from uzu_amd.serving import SequencePool
+    cfg, W, ms = models["a"]
+    m = ms[True]
+    m.set_sampling(None)
+    prompts = {"x": prompt(cfg, 3, 41), "y": prompt(cfg, 40, 42), "z": prompt(cfg, 17, 43)}
+    want = {k: O.greedy(cfg, W, p, 8) for k, p in prompts.items()}
+    stop = want["y"][4]
+    cut = lambda seq: seq[:seq.index(stop)] if stop in seq else seq
+    pool = SequencePool(m)
+    for _ in range(2):
+        got = pool.generate(prompts, max_tokens=8, stop_token_ids=[stop])
+        assert got == {k: cut(v) for k, v in want.items()}
+        assert not pool.live and len(pool.free) == 3
+    pool.close()

@@ -560,19 +560,16 @@ uzu_status s32_step_batch(uzu_hip_model* m, uzu_hip_state** states, uint32_t nse
         HIPCHK(hipMemcpyAsync(m->batch_tokens, pass_tok.data(), pass_tok.size() * 4, hipMemcpyHostToDevice, s));
         UZU_PROPAGATE(s32_pass(m, pass, m->batch_tokens, out_rows));
         for (size_t a = 0; a < pass.size(); ++a) {
-            const uint32_t qi = seq_lo + (uint32_t)a;
-            const bool finished = done[qi] == counts[qi];
             size_t srow = 0;
             bool do_sample = false;
             for (size_t b = 0; b < sample_seq.size(); ++b)
                 if (sample_seq[b] == a) srow = n_want_rows + b, do_sample = true;
-            (void)finished;
             UZU_PROPAGATE(sample_commit(m, pass[a].st, (uint32_t)srow, pass[a].count, do_sample));
         }
         HIPCHK(hipStreamSynchronize(s));
         for (size_t a = 0; a < pass.size(); ++a) state_set_length(m, pass[a].st, pass[a].start + pass[a].count);
-        for (size_t b = 0; b < n_want_rows; ++b)
-            HIPCHK(hipMemcpy(logits_out + (size_t)out_dst[b] * V, S.logits + b * V, (size_t)V * 4, hipMemcpyDeviceToHost));
+        // the wanted rows of a pass are consecutive entries of want_rows (both ascend): one copy
+        if (n_want_rows) HIPCHK(hipMemcpy(logits_out + (size_t)out_dst[0] * V, S.logits, n_want_rows * (size_t)V * 4, hipMemcpyDeviceToHost));
         for (size_t b = 0; b < sample_seq.size(); ++b) {
             const uint32_t qi = seq_lo + sample_seq[b];
             HIPCHK(hipMemcpy(sampled_out + qi, states[qi]->d_out_token, 4, hipMemcpyDeviceToHost));

@@ -246,3 +246,39 @@ def test_pool_generates_several_prompts_together(models):
         assert got == {k: cut(v) for k, v in want.items()}
         assert not pool.live and len(pool.free) == 3
     pool.close()
+
+
+@pytest.mark.parametrize("full", [True, False])
+def test_decode_graph_replays_equal_plain_launches(hip_ctx, tmp_path, full):
+    """The chained decode step is ONE captured hipGraph per state that reads its position from device memory.  Replayed in several calls, with eager batched
+    steps of OTHER states (which overwrite the model's pass tables) and synchronisations between them, every token and the logits after every call must equal
+    those of a model that decodes with plain launches."""
+    from uzu_amd.engine import MODEL_NO_GRAPH
+    cfg = cfg_b()
+    W = O.weights(cfg, 77)
+    O.write_model_dir(str(tmp_path / "m"), cfg, W)
+    bundle = loader.load_model_dir(str(tmp_path / "m"), max_context_length=256)
+    base = MODEL_BATCH(4) | (MODEL_FULL_F32 if full else 0)
+    graph, plain = HipModel(hip_ctx, bundle, base), HipModel(hip_ctx, bundle, base | MODEL_NO_GRAPH)
+    p, other = prompt(cfg, 70, 8), prompt(cfg, 33, 9)
+    firsts = [m.prefill(np.asarray(p, dtype=np.uint32)) for m in (graph, plain)]
+    assert firsts[0] == firsts[1]
+    side = [m.new_state() for m in (graph, plain)]
+    second = graph.new_state()
+    for call in range(4):
+        toks = [m.decode(5)[0] for m in (graph, plain)]
+        assert list(toks[0]) == list(toks[1]), call
+        assert np.array_equal(graph.read_logits_f32(), plain.read_logits_f32()), call
+        for m, st in zip((graph, plain), side):  # eager work on another state between the replays
+            m.step_batch([st], [other[call * 8:(call + 1) * 8]], [[7]])
+    # a second state of the same model gets a graph of its own; the first one's stays valid
+    graph.bind(second)
+    plain_second = plain.new_state()
+    plain.bind(plain_second)
+    a, b = graph.prefill(np.asarray(other, dtype=np.uint32)), plain.prefill(np.asarray(other, dtype=np.uint32))
+    assert a == b and list(graph.decode(6)[0]) == list(plain.decode(6)[0])
+    graph.bind(None)
+    plain.bind(None)
+    assert list(graph.decode(3)[0]) == list(plain.decode(3)[0]) and graph.context_length == 70 + 20 + 3
+    for m in (graph, plain):
+        m.close()

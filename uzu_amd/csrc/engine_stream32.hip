@@ -75,7 +75,7 @@ __global__ void s32_commit_kernel(uint32_t* ctx_len, uint32_t* tokens, const uin
 
 uzu_status need_f32(uzu_hip_model* m, size_t floats, float** out) {
     void* p = nullptr;
-    UZU_PROPAGATE(dev_alloc(m, floats * 4, &p, true));
+    UZU_PROPAGATE(dev_alloc(m, floats * 4, &p)); // scratch: every row a kernel reads was written earlier in the same pass (poison mode hands it out as NaNs)
     *out = (float*)p;
     return UZU_OK;
 }
@@ -445,19 +445,19 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
         void* q = nullptr;
         TRY(need_f32(m, R * w_moe, &S.moe_y1));
         TRY(need_f32(m, R * w_top * d, &S.moe_y2));
-        TRY(dev_alloc(m, R * w_top * 4, &q, true)); S.moe_perm = (uint32_t*)q;
-        TRY(dev_alloc(m, R * w_top * 4, &q, true)); S.moe_slot_pos = (uint32_t*)q;
-        TRY(dev_alloc(m, ((size_t)w_routed + 1) * 4, &q, true)); S.moe_offsets = (uint32_t*)q;
-        TRY(dev_alloc(m, ((size_t)w_routed + 1) * 4, &q, true)); S.moe_cursor = (uint32_t*)q;
+        TRY(dev_alloc(m, R * w_top * 4, &q)); S.moe_perm = (uint32_t*)q;
+        TRY(dev_alloc(m, R * w_top * 4, &q)); S.moe_slot_pos = (uint32_t*)q;
+        TRY(dev_alloc(m, ((size_t)w_routed + 1) * 4, &q)); S.moe_offsets = (uint32_t*)q;
+        TRY(dev_alloc(m, ((size_t)w_routed + 1) * 4, &q)); S.moe_cursor = (uint32_t*)q;
     }
     void* p = nullptr;
-    TRY(dev_alloc(m, R * w_top * 4, &p, true)); S.moe_ids = (int32_t*)p;
-    TRY(dev_alloc(m, S.max_seqs * sizeof(k::SeqSpan), &p, true)); S.d_spans = (k::SeqSpan*)p;
-    TRY(dev_alloc(m, R * 4, &p, true)); S.d_row_seq = (uint32_t*)p;
-    TRY(dev_alloc(m, R * 4, &p, true)); S.d_out_rows = (uint32_t*)p;
-    TRY(dev_alloc(m, (size_t)nl * S.max_seqs * sizeof(void*), &p, true)); S.d_cache_ptrs = (void**)p;
-    TRY(dev_alloc(m, (size_t)nl * S.max_seqs * sizeof(float*), &p, true)); S.d_shift_ptrs = (float**)p;
-    TRY(dev_alloc(m, R * 4, &p, true)); m->batch_tokens = (uint32_t*)p;
+    TRY(dev_alloc(m, R * w_top * 4, &p)); S.moe_ids = (int32_t*)p;
+    TRY(dev_alloc(m, S.max_seqs * sizeof(k::SeqSpan), &p)); S.d_spans = (k::SeqSpan*)p;
+    TRY(dev_alloc(m, R * 4, &p)); S.d_row_seq = (uint32_t*)p;
+    TRY(dev_alloc(m, R * 4, &p)); S.d_out_rows = (uint32_t*)p;
+    TRY(dev_alloc(m, (size_t)nl * S.max_seqs * sizeof(void*), &p)); S.d_cache_ptrs = (void**)p;
+    TRY(dev_alloc(m, (size_t)nl * S.max_seqs * sizeof(float*), &p)); S.d_shift_ptrs = (float**)p;
+    TRY(dev_alloc(m, R * 4, &p)); m->batch_tokens = (uint32_t*)p;
     if (flags & UZU_MODEL_DEBUG_TAPS) TRY(need_f32(m, (size_t)nl * R * d, &S.taps));
     {
         uint32_t hmax = 0;

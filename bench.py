@@ -11,6 +11,9 @@ and the synthetic prompt of SURVEY.md §8d; all inputs are resident in HBM when 
 Prints ONE JSON line on rank 0 (contract in the task statement) with two extra objects:
   roofline     -- the dominant kernel (the int4 GEMV family) : algorithmic bytes / HIP-event time, vs 8 TB/s HBM
   cpu_baseline -- the CPU oracle (port of the reference's single-threaded CPU backend) timed on this host
+
+Side runs (their own JSON line, never the headline): --config c3|c4|c5, --exact, and --design lazolix (prefill / chained decode / batched decode of the
+f32-stream design at real layer sizes beside the closest bf16-stream model).
 """
 import argparse
 import dataclasses

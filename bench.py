@@ -13,7 +13,7 @@ Prints ONE JSON line on rank 0 (contract in the task statement) with two extra o
   cpu_baseline -- the CPU oracle (port of the reference's single-threaded CPU backend) timed on this host
 
 Side runs (their own JSON line, never the headline): --config c3|c4|c5, --exact, and --design lazolix (prefill / chained decode / batched decode of the
-f32-stream design at real layer sizes beside the closest bf16-stream model).
+f32-stream design at real layer sizes beside the closest bf16-stream model of the engine).
 """
 import argparse
 import dataclasses

@@ -80,7 +80,8 @@ typedef struct {
 /* config/normalization.rs:10-18 + tensor `scales` f32 [dim] (encodable_block/normalization.rs:67-74) */
 typedef enum {
     UZU_NORM_STATISTICS = 0,   /* RMS / mean-variance normalisation (the reference's Normalization) */
-    UZU_NORM_DYNAMIC_TANH = 1  /* no statistics: y = tanh(alpha * x) * scales + biases, element by element (f32-stream designs) */
+    UZU_NORM_DYNAMIC_TANH = 1, /* no statistics: y = tanh(alpha * x) * scales + biases, element by element (f32-stream designs) */
+    UZU_NORM_RMS_SCALAR = 2    /* y = alpha * x / sqrt(mean(x^2) + epsilon): RMS norm with ONE gain for all coordinates (alpha; no scales tensor) (f32-stream designs) */
 } uzu_norm_kind;
 typedef struct {
     uint32_t present;       /* 0 => this optional norm is absent */
@@ -91,7 +92,7 @@ typedef struct {
     float scale_offset;     /* Option<f32>::unwrap_or(0.0) */
     const float* scales;    /* f32 [dim] or NULL (has_scale == false) */
     const float* biases;    /* f32 [dim] or NULL */
-    float alpha;            /* UZU_NORM_DYNAMIC_TANH: the scalar inside the tanh */
+    float alpha;            /* UZU_NORM_DYNAMIC_TANH: the scalar inside the tanh; UZU_NORM_RMS_SCALAR: the gain */
     uint32_t reserved;
 } uzu_norm_desc;
 
@@ -103,7 +104,13 @@ typedef enum {
      * attention fields: num_heads, head_dim (query / key width per head), attention_scale, sliding_window_size, has_sinks / sinks, is_kv_sharing +
      * kv_source_layer_index (the sharing layer reads the source layer's cached latents through its OWN up projections), qkv_projection (queries only,
      * n = heads * head_dim), out_projection (k = heads * value_head_dim); and the latent_* fields at the end of uzu_layer_desc. */
-    UZU_MIXER_LATENT_ATTENTION = 2
+    UZU_MIXER_LATENT_ATTENTION = 2,
+    /* Retention (f32-stream designs): linear attention with a fixed decay per head and neither softmax nor denominator.  Per head a: S_t = decay[a] S_(t-1) +
+     * k_t v_t^T (f32 [head_dim, value_head_dim], the sequence state, zero at position 0), o_t = S_t^T q_t; every head's o_t is divided by its root mean square
+     * (head_norm_epsilon, no weights), the heads are concatenated, multiplied by silu(gate h) and projected.  q and k are rotated (use_rope) and k is multiplied
+     * by key_scale behind its rotation.  Fields: num_heads, head_dim, value_head_dim, retention_decay, qkv_projection (rows: queries | keys | values | gate,
+     * n = 2 heads head_dim + 2 heads value_head_dim), out_projection (k = heads * value_head_dim). */
+    UZU_MIXER_RETENTION = 3
 } uzu_mixer_kind;
 
 /* config/rope/*.rs -- every AnyRoPEConfig variant (encodable_block/mixer/attention/rope.rs:13-114) */
@@ -154,6 +161,11 @@ typedef struct {
     uint32_t routing;              /* uzu_moe_routing; 0 = the reference's top-k of the logits */
     uint32_t num_identity_experts;
     const float* selection_bias;   /* f32 [routed + identity]: added to the scores for the choice only */
+    /* expert = down(act(gate) * (up + up_offset)) with the clipping above applied first; 0 = the plain gated product.  In an f32-stream design top-k routing
+     * (routing == 0) reads router_biases (bf16 [E], optional), takes the num_active_experts largest logits (ties: the lower index) and, with router_renorm, the
+     * softmax over the winners' logits as weights; the experts have no biases. */
+    float up_offset;
+    uint32_t reserved;
 } uzu_moe_desc;
 typedef enum { UZU_MOE_ROUTE_TOPK_LOGITS = 0, UZU_MOE_ROUTE_SCORES = 1 } uzu_moe_routing;
 
@@ -246,7 +258,21 @@ typedef struct {
     uint32_t num_depth_weights;  /* l + 2 on layer l */
     uint32_t mlp_plain;          /* dense MLP without a gate: down(act(up x + b) ) + b, up_projection.n == hidden_dim */
     uint32_t no_mlp;             /* the layer ends behind its mixer */
+    /* Parallel block: the mixer and the MLP both read pre_mixer_norm's rows and the layer is x <- x + (mixer(h) + mlp(h)); there is no pre_mlp_norm. */
+    uint32_t parallel_block;
+    /* UZU_MIXER_ATTENTION in an f32-stream design: grouped heads (num_heads queries on num_groups key / value heads, query head a reads head a / (heads / groups)),
+     * key width head_dim and value width value_head_dim, qkv_projection rows = queries | keys | values (n = heads head_dim + groups (head_dim + value_head_dim);
+     * a sharing layer: queries only) with out_biases, rotation of the first rope dimensions of queries and keys (use_rope, rope_index), scores
+     * attention_scale <q, k>, then the soft cap, causal sliding window (sliding_window_size, 0 = all earlier positions), softmax with per-head sink logits in the
+     * denominator (has_sinks + sinks, or unit_sink), out_projection.k = heads * value_head_dim.  The cache keeps rotated keys and values per position;
+     * is_kv_sharing reads the source layer's cache with this layer's own queries, mask and constants. */
+    float score_soft_cap;        /* s <- cap * tanh(s / cap); 0 = none */
+    uint32_t unit_sink;          /* one more term exp(0) in every softmax denominator (a sink with logit 0 and no value) */
+    float key_scale;             /* keys are multiplied by it behind their rotation; 0 = 1 */
+    float head_norm_epsilon;     /* UZU_MIXER_RETENTION: epsilon of the per-head RMS division */
+    const float* retention_decay; /* UZU_MIXER_RETENTION: f32 [num_heads] */
     uint32_t reserved4;
+    uint32_t reserved6;
 } uzu_layer_desc;
 
 typedef struct {

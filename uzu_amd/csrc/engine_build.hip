@@ -106,8 +106,8 @@ uzu_status state_build(uzu_hip_model* m, uzu_hip_state** out) {
     for (size_t l = 0; l < m->layers.size(); ++l) {
         const uzu_layer_desc& h = m->layers[l].d;
         void* p = nullptr;
-        if (h.mixer_kind == UZU_MIXER_LATENT_ATTENTION) {
-            if (r == UZU_OK) r = s32_state_layer(m, st, (uint32_t)l); // latent cache (unless shared) + the token shift's row
+        if (m->s32) {
+            if (r == UZU_OK) r = s32_state_layer(m, st, (uint32_t)l); // latent / key-value cache (unless shared), retention state, the token shift's row
         } else if (h.mixer_kind == UZU_MIXER_ATTENTION && h.is_kv_sharing) {
             // TransformerLayerStateType::Shared(kv_source_layer_index) (transformer.rs:205-216): no state of its own
         } else if (h.mixer_kind == UZU_MIXER_ATTENTION) {
@@ -281,7 +281,7 @@ void rope_tables(const uzu_rope_desc& r, uint32_t n_pos, std::vector<float>& cos
             if (r.truncate) low = floor(low), high = ceil(high);
             const float low_f = (float)(low > 0.0 ? low : 0.0);
             float high_f = (float)(high < (double)(r.head_dim - 1) ? high : (double)(r.head_dim - 1));
-            if (low_f == high_f) high_f += 0.001f;
+            if (high_f - low_f < 0.001f) high_f = low_f + 0.001f; // (the reference's guard for low == high, also where the clamps cross)
             float ramp = ((float)pair_index - low_f) / (high_f - low_f);
             ramp = ramp < 0.0f ? 0.0f : (ramp > 1.0f ? 1.0f : ramp);
             const float smoothing_factor = 1.0f - ramp;
@@ -326,7 +326,8 @@ uzu_status uzu_hip_model_create_tp(uzu_hip_context* ctx, const uzu_model_desc* d
     }
     UZU_UNSUPPORTED(flags & UZU_MODEL_FULL_F32, "model_create: UZU_MODEL_FULL_F32 is a precision of the f32-stream designs; this model's stream is bf16");
     for (uint32_t l = 0; l < desc->num_layers; ++l)
-        UZU_UNSUPPORTED(desc->layers[l].mixer_kind == UZU_MIXER_LATENT_ATTENTION || desc->layers[l].token_shift || desc->layers[l].depth_weights || desc->layers[l].mlp_plain ||
+        UZU_UNSUPPORTED(desc->layers[l].mixer_kind == UZU_MIXER_LATENT_ATTENTION || desc->layers[l].mixer_kind == UZU_MIXER_RETENTION || desc->layers[l].parallel_block ||
+                        desc->layers[l].score_soft_cap != 0.0f || desc->layers[l].unit_sink || desc->layers[l].key_scale != 0.0f || desc->layers[l].token_shift || desc->layers[l].depth_weights || desc->layers[l].mlp_plain ||
                         desc->layers[l].no_mlp || desc->layers[l].pre_mixer_norm.kind != UZU_NORM_STATISTICS || desc->layers[l].pre_mlp_norm.kind != UZU_NORM_STATISTICS ||
                         (desc->layers[l].mlp_kind == UZU_MLP_MOE && desc->layers[l].moe.routing != UZU_MOE_ROUTE_TOPK_LOGITS),
                         "model_create: layer %u uses a mechanism of the f32-stream designs (set uzu_model_desc::f32_stream)", l);

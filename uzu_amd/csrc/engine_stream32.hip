@@ -10,6 +10,12 @@
 // latent cache and the attention core address each row's own sequence through pointer tables built per pass.  A prompt longer than one pass (m->chunk rows)
 // continues in the next pass from the state the previous one left: the cache rows and the last normalised row per layer.
 //
+// Next to those the encoder carries the mechanisms of designs with rotated attention and recurrent layers (second family: Relulix): RMS norms with one gain,
+// parallel blocks (mixer and MLP read the same normalised rows, one residual add), attention over a per-position cache of rotated keys and values (grouped
+// heads, biases, partial rotation with scaled frequencies, soft-capped scores, sliding window, a unit sink; k_window_attention.hip), retention layers with an
+// f32 state per sequence (k_retention.hip), top-k routed experts with clamped gates, a scaled embedding and an untied read-out.  Each is chosen per layer by the
+// description's fields, so a model may mix them.
+//
 // Precisions: `bf16_products` (default) rounds the activation operand of every matrix product to bf16 and keeps the latent cache in bf16; UZU_MODEL_FULL_F32
 // makes every product a true f32 product and the cache f32.  Everything else is f32 either way.
 #include <algorithm>
@@ -36,13 +42,15 @@ struct Stream32 {
     size_t logit_rows = 0;
     k::SeqSpan* d_spans = nullptr;
     uint32_t *d_row_seq = nullptr, *d_out_rows = nullptr;
-    void** d_cache_ptrs = nullptr;  // [layers][max_seqs]
+    void** d_cache_ptrs = nullptr;  // [layers][max_seqs]: latent rows / key rows / the retention state
+    void** d_cache2_ptrs = nullptr; // [layers][max_seqs]: value rows
     float** d_shift_ptrs = nullptr; // [layers][max_seqs]
     struct Layer {
         uint16_t* up_keys_t = nullptr; // bf16 [heads][rank][head_dim]: W_up_k of a head transposed, so that folding it into the query is an ordinary product
         float* sinks = nullptr;        // f32 [heads]
         float *token_shift = nullptr, *depth_weights = nullptr, *selection_bias = nullptr;
         float alpha1 = 0.f, alpha2 = 0.f;
+        float* decay = nullptr; // retention: f32 [heads]
     };
     std::vector<Layer> layers;
     float alpha_out = 0.f;
@@ -100,6 +108,27 @@ void run_linear(Enc& e, const k::LinearF32Params& p) {
     e.run(r, variant, k::linear_f32_bytes(p));
 }
 
+// a norm of the stream's rows by its kind; row_index: a gather of the rows (the read-out)
+void run_norm(Enc& e, const DNorm& N, uint32_t kind, float alpha, const float* x, float* out, uint32_t rows, uint32_t d, const uint32_t* row_index) {
+    hipStream_t s = e.s;
+    if (kind == UZU_NORM_RMS_SCALAR) {
+        RUN("rms_norm_rows", (size_t)rows * d * 8, k::rms_norm_rows(s, x, out, nullptr, alpha, N.eps, row_index, rows, d));
+        return;
+    }
+    k::DynTanhParams np{};
+    np.x = x, np.out = out, np.scales = N.scales, np.biases = N.biases, np.alpha = alpha, np.row_index = row_index, np.rows = rows, np.d = d;
+    RUN("dyn_tanh_norm", (size_t)rows * d * 8, k::dyn_tanh_norm(s, np));
+}
+
+k::ExpertAct expert_act(const uzu_moe_desc& M) {
+    k::ExpertAct a;
+    a.alpha = M.silu_alpha != 0.0f ? M.silu_alpha : 1.0f;
+    if (M.gate_clip_min != 0.0f || M.gate_clip_max != 0.0f) a.gate_min = M.gate_clip_min, a.gate_max = M.gate_clip_max; // (all zero: a description that never set them)
+    if (M.up_clip_min != 0.0f || M.up_clip_max != 0.0f) a.up_min = M.up_clip_min, a.up_max = M.up_clip_max;
+    a.up_offset = M.up_offset;
+    return a;
+}
+
 // The tables of a pass over `seqs`: spans, row -> sequence, per-layer cache / shift-state pointers, the rows whose logits are wanted.
 uzu_status s32_upload_tables(uzu_hip_model* m, const std::vector<PassSeq>& seqs, const std::vector<uint32_t>& out_rows) {
     Stream32& S = *m->s32;
@@ -116,20 +145,25 @@ uzu_status s32_upload_tables(uzu_hip_model* m, const std::vector<PassSeq>& seqs,
         rows += seqs[i].count;
     }
     UZU_REQUIRE(rows <= S.max_rows, "engine: a pass of %u rows (at most %u)", rows, S.max_rows);
-    std::vector<void*> cache_ptrs((size_t)nl * S.max_seqs, nullptr);
+    std::vector<void*> cache_ptrs((size_t)nl * S.max_seqs, nullptr), cache2_ptrs((size_t)nl * S.max_seqs, nullptr);
     std::vector<float*> shift_ptrs((size_t)nl * S.max_seqs, nullptr);
     for (uint32_t l = 0; l < nl; ++l) {
         const uzu_layer_desc& h = m->layers[l].d;
         const uint32_t src = h.is_kv_sharing ? h.kv_source_layer_index : l;
         for (uint32_t i = 0; i < nseq; ++i) {
-            cache_ptrs[(size_t)l * S.max_seqs + i] = seqs[i].st->layers[src].latent;
-            shift_ptrs[(size_t)l * S.max_seqs + i] = seqs[i].st->layers[l].shift_prev;
+            const uzu_hip_state::Layer& own = seqs[i].st->layers[src];
+            const size_t at = (size_t)l * S.max_seqs + i;
+            if (h.mixer_kind == UZU_MIXER_ATTENTION) cache_ptrs[at] = own.cache_k, cache2_ptrs[at] = own.cache_v;
+            else if (h.mixer_kind == UZU_MIXER_RETENTION) cache_ptrs[at] = own.ret_state;
+            else cache_ptrs[at] = own.latent;
+            shift_ptrs[at] = seqs[i].st->layers[l].shift_prev;
         }
     }
     // (pageable sources: the copies have left the host buffers when the calls return)
     HIPCHK(hipMemcpyAsync(S.d_spans, spans.data(), spans.size() * sizeof(k::SeqSpan), hipMemcpyHostToDevice, s));
     HIPCHK(hipMemcpyAsync(S.d_row_seq, row_seq.data(), row_seq.size() * 4, hipMemcpyHostToDevice, s));
     HIPCHK(hipMemcpyAsync(S.d_cache_ptrs, cache_ptrs.data(), cache_ptrs.size() * sizeof(void*), hipMemcpyHostToDevice, s));
+    HIPCHK(hipMemcpyAsync(S.d_cache2_ptrs, cache2_ptrs.data(), cache2_ptrs.size() * sizeof(void*), hipMemcpyHostToDevice, s));
     HIPCHK(hipMemcpyAsync(S.d_shift_ptrs, shift_ptrs.data(), shift_ptrs.size() * sizeof(float*), hipMemcpyHostToDevice, s));
     if (!out_rows.empty()) HIPCHK(hipMemcpyAsync(S.d_out_rows, out_rows.data(), out_rows.size() * 4, hipMemcpyHostToDevice, s));
     return UZU_OK;
@@ -149,7 +183,7 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
     for (uint32_t c : counts) rows += c;
     const size_t slot_stride = (size_t)S.max_rows * d;
     const uint32_t bf = S.full_f32 ? 0u : 1u;
-    RUN("embed_rows_f32", (size_t)rows * d * 6, k::embed_rows_f32(s, d_tokens, (const uint16_t*)m->embedding.w, S.slots, rows, m->d.vocab_size, d));
+    RUN("embed_rows_f32", (size_t)rows * d * 6, k::embed_rows_f32(s, d_tokens, (const uint16_t*)m->embedding.w, S.slots, rows, m->d.vocab_size, d, m->d.input_scale));
     const float* cur = S.slots; // what the layer about to run reads: X_0, then the depth mix of the layer before
     for (uint32_t l = 0; l < nl; ++l) {
         DLayer& L = m->layers[l];
@@ -157,14 +191,43 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
         const uzu_layer_desc& h = L.d;
         float* slot = S.slots + (size_t)(l + 1) * slot_stride; // X_(l+1): the layer's own result
         void* const* caches = S.d_cache_ptrs + (size_t)l * S.max_seqs;
-        {   // pre-mixer norm + token shift
+        if (h.pre_mixer_norm.kind == UZU_NORM_RMS_SCALAR) {
+            run_norm(e, L.pre_mixer, h.pre_mixer_norm.kind, X.alpha1, cur, S.normed, rows, d, nullptr);
+        } else { // dynamic-tanh norm + token shift
             k::DynTanhParams np{};
             np.x = cur, np.out = S.normed, np.scales = L.pre_mixer.scales, np.biases = L.pre_mixer.biases, np.alpha = X.alpha1, np.shift = X.token_shift;
             np.spans = S.d_spans, np.row_seq = S.d_row_seq, np.prev = S.d_shift_ptrs + (size_t)l * S.max_seqs, np.rows = rows, np.d = d;
             RUN("dyn_tanh_norm+shift", (size_t)rows * d * 8, k::dyn_tanh_norm(s, np));
         }
         const uint32_t H = h.num_heads, hd = h.head_dim, vd = h.value_head_dim, rank = h.latent_rank;
-        run_linear(e, lin(S, L.qkv, S.normed, S.q, rows));
+        run_linear(e, lin(S, L.qkv, S.normed, S.q, rows)); // the packed projection of the mixer (queries first)
+        if (h.mixer_kind == UZU_MIXER_ATTENTION) {
+            const uint32_t G = h.num_groups, ldq = L.qkv.n;
+            void* const* vcaches = S.d_cache2_ptrs + (size_t)l * S.max_seqs;
+            k::RopeAppendParams rp{};
+            rp.qkv = S.q, rp.ld = ldq, rp.k_col = H * hd, rp.v_col = H * hd + G * hd, rp.heads = H, rp.kv_heads = h.is_kv_sharing ? 0u : G, rp.dim = hd, rp.vdim = vd;
+            rp.rope_dim = h.use_rope ? L.rope_dim : 0u, rp.cosines = L.rope_cos, rp.sines = L.rope_sin, rp.key_scale = h.key_scale != 0.0f ? h.key_scale : 1.0f;
+            rp.key_caches = caches, rp.value_caches = vcaches, rp.cache_bf16 = bf, rp.spans = S.d_spans, rp.row_seq = S.d_row_seq, rp.rows = rows;
+            RUN("rope_append", (size_t)rows * ldq * 8, k::rope_append(s, rp));
+            k::WindowAttentionParams ap{};
+            ap.q = S.q, ap.ldq = ldq, ap.out = S.attn, ap.key_caches = caches, ap.value_caches = vcaches, ap.cache_bf16 = bf, ap.sinks = X.sinks, ap.spans = S.d_spans;
+            ap.row_seq = S.d_row_seq, ap.rows = rows, ap.heads = H, ap.kv_heads = G, ap.dim = hd, ap.vdim = vd, ap.window = h.sliding_window_size;
+            ap.scale = h.attention_scale != 0.0f ? h.attention_scale : 1.0f / sqrtf((float)hd), ap.soft_cap = h.score_soft_cap, ap.nseq = nseq;
+            for (uint32_t i = 0; i < nseq; ++i) ap.tiles += (counts[i] + 63) / 64;
+            RUN("window_attention", (size_t)rows * H * (hd + vd) * 4, k::window_attention(s, ap));
+        } else if (h.mixer_kind == UZU_MIXER_RETENTION) {
+            const uint32_t ldq = L.qkv.n; // queries | keys | values | gate
+            k::RopeAppendParams rp{};
+            rp.qkv = S.q, rp.ld = ldq, rp.k_col = H * hd, rp.v_col = 2 * H * hd, rp.heads = H, rp.kv_heads = H, rp.dim = hd, rp.vdim = vd;
+            rp.rope_dim = h.use_rope ? L.rope_dim : 0u, rp.cosines = L.rope_cos, rp.sines = L.rope_sin, rp.key_scale = h.key_scale != 0.0f ? h.key_scale : 1.0f;
+            rp.spans = S.d_spans, rp.row_seq = S.d_row_seq, rp.rows = rows;
+            RUN("rope_append", (size_t)rows * 2 * H * hd * 8, k::rope_append(s, rp));
+            k::RetentionParams tp{};
+            tp.qkv = S.q, tp.ld = ldq, tp.q_col = 0, tp.k_col = H * hd, tp.v_col = 2 * H * hd, tp.out = S.attn, tp.states = (float* const*)caches, tp.decay = X.decay;
+            tp.spans = S.d_spans, tp.nseq = nseq, tp.rows = rows, tp.heads = H, tp.dim = hd, tp.vdim = vd;
+            RUN("retention", (size_t)rows * ldq * 4 + (size_t)nseq * H * hd * vd * 8, k::retention(s, tp));
+            RUN("head_rms_gate", (size_t)rows * H * vd * 12, k::head_rms_gate(s, S.attn, S.q + 2 * H * hd + H * vd, ldq, h.head_norm_epsilon, rows, H, vd));
+        } else {
         if (!h.is_kv_sharing) {
             run_linear(e, lin(S, L.lat_down, S.normed, S.ckv, rows));
             RUN("latent_norm_append", (size_t)rows * rank * 6,
@@ -194,28 +257,33 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
             p.x_batch = rank, p.w_batch = (size_t)vd * rank, p.y_batch = vd, p.bf16_products = bf;
             run_linear(e, p);
         }
+        } // latent attention
         {   // X_(l+1) = input + out projection
             k::LinearF32Params p = lin(S, L.out, S.attn, slot, rows);
             p.residual = cur, p.ldr = d;
             run_linear(e, p);
         }
         if (!h.no_mlp) {
-            k::DynTanhParams np{};
-            np.x = slot, np.out = S.normed, np.scales = L.pre_mlp.scales, np.biases = L.pre_mlp.biases, np.alpha = X.alpha2, np.rows = rows, np.d = d;
-            RUN("dyn_tanh_norm", (size_t)rows * d * 8, k::dyn_tanh_norm(s, np));
+            // a parallel block's MLP reads the rows the mixer read (still in S.normed) and adds to the same sum; otherwise the MLP has its own norm of the sum so far
+            if (!h.parallel_block) run_norm(e, L.pre_mlp, h.pre_mlp_norm.kind, X.alpha2, slot, S.normed, rows, d, nullptr);
             if (h.mlp_kind == UZU_MLP_MOE) {
                 const uzu_moe_desc& M = h.moe;
                 const uint32_t E = M.num_routed_experts, top = M.num_active_experts, ff = M.expert_hidden_dim;
-                RUN("moe_route_scores", (size_t)(E + M.num_identity_experts) * d * 2,
-                    k::moe_route_scores(s, S.normed, L.moe.router_weights, X.selection_bias, S.moe_ids, S.moe_w, rows, d, E + M.num_identity_experts, top));
+                const k::ExpertAct act = expert_act(M);
+                if (M.routing == UZU_MOE_ROUTE_SCORES) {
+                    RUN("moe_route_scores", (size_t)(E + M.num_identity_experts) * d * 2,
+                        k::moe_route_scores(s, S.normed, L.moe.router_weights, X.selection_bias, S.moe_ids, S.moe_w, rows, d, E + M.num_identity_experts, top));
+                } else {
+                    RUN("moe_route_topk", (size_t)E * d * 2, k::moe_route_topk(s, S.normed, L.moe.router_weights, L.moe.router_biases, S.moe_ids, S.moe_w, rows, d, E, top, M.router_renorm));
+                }
                 k::MoeGroupedParams gp{};
                 gp.x = S.normed, gp.ids = S.moe_ids, gp.weights = S.moe_w, gp.w13 = L.moe.w13, gp.w2 = L.moe.w2, gp.residual = slot, gp.y = slot, gp.y1 = S.moe_y1, gp.hidden = S.hid;
                 gp.y2 = S.moe_y2, gp.perm = S.moe_perm, gp.slot_pos = S.moe_slot_pos, gp.offsets = S.moe_offsets, gp.cursor = S.moe_cursor;
-                gp.rows = rows, gp.d = d, gp.ff = ff, gp.routed = E, gp.top = top;
+                gp.rows = rows, gp.d = d, gp.ff = ff, gp.routed = E, gp.top = top, gp.act = act;
                 if (bf && k::moe_experts_grouped_supported(gp)) { // prefill-sized: buckets per expert through the matrix-core linear
                     RUN("moe_experts_grouped", (size_t)E * 3 * ff * d * 2 + (size_t)rows * top * (3 * ff + 2 * d) * 4, k::moe_experts_grouped(s, gp));
                 } else {
-                    RUN("moe_experts_gate_up", (size_t)rows * top * 2 * ff * d * 2, k::moe_experts_gate_up(s, S.normed, S.moe_ids, L.moe.w13, S.hid, rows, d, ff, E, top, bf));
+                    RUN("moe_experts_gate_up", (size_t)rows * top * 2 * ff * d * 2, k::moe_experts_gate_up(s, S.normed, S.moe_ids, L.moe.w13, S.hid, rows, d, ff, E, top, bf, act));
                     RUN("moe_experts_down_combine", (size_t)rows * top * ff * d * 2,
                         k::moe_experts_down_combine(s, S.hid, S.normed, S.moe_ids, S.moe_w, L.moe.w2, slot, slot, rows, d, ff, E, top, bf));
                 }
@@ -239,11 +307,8 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
     S.tap_rows = rows;
     S.last_logit_rows = 0;
     if (n_out) {
-        k::DynTanhParams np{};
-        np.x = cur, np.out = S.out_normed, np.scales = m->output_norm.scales, np.biases = m->output_norm.biases, np.alpha = S.alpha_out, np.row_index = S.d_out_rows;
-        np.rows = n_out, np.d = d;
-        RUN("dyn_tanh_norm", (size_t)n_out * d * 8, k::dyn_tanh_norm(s, np));
-        run_linear(e, lin(S, m->embedding, S.out_normed, S.logits, n_out));
+        run_norm(e, m->output_norm, m->d.output_norm.kind, S.alpha_out, cur, S.out_normed, n_out, d, S.d_out_rows);
+        run_linear(e, lin(S, m->d.tied_embeddings ? m->embedding : m->output_embedding, S.out_normed, S.logits, n_out));
         S.last_logit_rows = n_out;
     }
     if (e.st != UZU_OK) return e.st;
@@ -313,37 +378,76 @@ uzu_status sample_commit(uzu_hip_model* m, uzu_hip_state* st, uint32_t logit_row
 
 uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t flags, uzu_hip_model** out) {
     const uint32_t d = desc->model_dim, nl = desc->num_layers;
-    UZU_REQUIRE(desc->tied_embeddings && desc->embedding.method == UZU_QUANT_NONE && desc->embedding.weights && desc->embedding.n == desc->vocab_size && desc->embedding.k == d,
-                "model_create: an f32-stream design reads out through its full-precision embedding table [vocab, model_dim]");
-    UZU_REQUIRE(desc->output_norm.present && desc->output_norm.kind == UZU_NORM_DYNAMIC_TANH && desc->output_norm.scales, "model_create: an f32-stream design ends in a dynamic-tanh norm");
-    UZU_UNSUPPORTED(desc->has_ple || desc->embedding_norm.present || desc->num_ropes || desc->logit_soft_cap != 0.0f || desc->logit_scale != 1.0f || desc->input_scale != 1.0f,
+    UZU_REQUIRE(desc->embedding.method == UZU_QUANT_NONE && desc->embedding.weights && desc->embedding.n == desc->vocab_size && desc->embedding.k == d,
+                "model_create: an f32-stream design embeds through a full-precision table [vocab, model_dim]");
+    UZU_REQUIRE(desc->tied_embeddings || (desc->output_embedding.method == UZU_QUANT_NONE && desc->output_embedding.weights && desc->output_embedding.n == desc->vocab_size &&
+                                          desc->output_embedding.k == d && !desc->output_embedding.out_biases),
+                "model_create: an untied read-out of an f32-stream design is a full-precision matrix [vocab, model_dim]");
+    auto norm_ok = [](const uzu_norm_desc& n) { return n.present && ((n.kind == UZU_NORM_DYNAMIC_TANH && n.scales) || n.kind == UZU_NORM_RMS_SCALAR); };
+    UZU_REQUIRE(norm_ok(desc->output_norm), "model_create: an f32-stream design ends in a dynamic-tanh norm or an RMS norm with one gain");
+    UZU_UNSUPPORTED(desc->has_ple || desc->embedding_norm.present || desc->logit_soft_cap != 0.0f || desc->logit_scale != 1.0f,
                     "model_create: decoder options of the bf16-stream families on an f32-stream design");
     auto full = [](const uzu_linear_desc& L, uint32_t n, uint32_t kk) { return L.weights && L.method == UZU_QUANT_NONE && L.n == n && L.k == kk && !L.input_signs && !L.output_signs && !L.lora_rank; };
     for (uint32_t l = 0; l < nl; ++l) {
         const uzu_layer_desc& h = desc->layers[l];
-        UZU_UNSUPPORTED(h.mixer_kind != UZU_MIXER_LATENT_ATTENTION, "model_create: layer %u: an f32-stream design's mixer is latent attention", l);
-        UZU_REQUIRE(h.pre_mixer_norm.present && h.pre_mixer_norm.kind == UZU_NORM_DYNAMIC_TANH && h.pre_mixer_norm.scales, "model_create: layer %u needs a dynamic-tanh pre-mixer norm", l);
-        UZU_REQUIRE(h.num_heads && h.head_dim && h.value_head_dim && h.latent_rank && h.latent_rank <= k::kLatentMaxRank, "model_create: layer %u: heads / head_dim / value_head_dim / latent_rank (<= %u)",
-                    l, k::kLatentMaxRank);
-        UZU_REQUIRE(full(h.qkv_projection, h.num_heads * h.head_dim, d) && full(h.out_projection, d, h.num_heads * h.value_head_dim) &&
-                    full(h.latent_up_keys, h.num_heads * h.head_dim, h.latent_rank) && full(h.latent_up_values, h.num_heads * h.value_head_dim, h.latent_rank),
-                    "model_create: layer %u: query / out / latent up projections must be full-precision matrices of the configured shapes", l);
-        if (h.is_kv_sharing) {
-            UZU_REQUIRE(h.kv_source_layer_index < l, "model_create: layer %u shares the latents of layer %u, which does not precede it", l, h.kv_source_layer_index);
-            const uzu_layer_desc& src = desc->layers[h.kv_source_layer_index];
-            UZU_REQUIRE(!src.is_kv_sharing && src.latent_rank == h.latent_rank, "model_create: layer %u: the source layer %u must own latents of the same rank", l, h.kv_source_layer_index);
+        UZU_UNSUPPORTED(h.mixer_kind != UZU_MIXER_LATENT_ATTENTION && h.mixer_kind != UZU_MIXER_ATTENTION && h.mixer_kind != UZU_MIXER_RETENTION,
+                        "model_create: layer %u: an f32-stream design's mixer is latent attention, attention over cached keys and values, or retention", l);
+        UZU_REQUIRE(norm_ok(h.pre_mixer_norm), "model_create: layer %u needs a dynamic-tanh or one-gain RMS pre-mixer norm", l);
+        UZU_UNSUPPORTED(h.token_shift && h.pre_mixer_norm.kind != UZU_NORM_DYNAMIC_TANH, "model_create: layer %u: the token shift follows a dynamic-tanh norm", l);
+        UZU_REQUIRE(h.num_heads && h.head_dim && h.value_head_dim, "model_create: layer %u: heads / head_dim / value_head_dim", l);
+        UZU_REQUIRE(full(h.out_projection, d, h.num_heads * h.value_head_dim), "model_create: layer %u: the out projection must be a full-precision matrix [model_dim, heads * value_head_dim]", l);
+        if (h.use_rope) {
+            const uzu_rope_desc& R = desc->num_ropes ? desc->ropes[h.rope_index < desc->num_ropes ? h.rope_index : 0] : desc->rope;
+            UZU_REQUIRE(h.mixer_kind != UZU_MIXER_LATENT_ATTENTION && (!desc->num_ropes || h.rope_index < desc->num_ropes) && R.kind != UZU_ROPE_NONE && R.head_dim && R.head_dim % 2 == 0 &&
+                        R.head_dim <= h.head_dim, "model_create: layer %u: its rotation must turn an even number of at most head_dim coordinates", l);
+        }
+        if (h.mixer_kind == UZU_MIXER_LATENT_ATTENTION) {
+            UZU_REQUIRE(h.latent_rank && h.latent_rank <= k::kLatentMaxRank, "model_create: layer %u: latent_rank (<= %u)", l, k::kLatentMaxRank);
+            UZU_REQUIRE(full(h.qkv_projection, h.num_heads * h.head_dim, d) && full(h.latent_up_keys, h.num_heads * h.head_dim, h.latent_rank) &&
+                        full(h.latent_up_values, h.num_heads * h.value_head_dim, h.latent_rank),
+                        "model_create: layer %u: query / latent up projections must be full-precision matrices of the configured shapes", l);
+            if (h.is_kv_sharing) {
+                UZU_REQUIRE(h.kv_source_layer_index < l, "model_create: layer %u shares the latents of layer %u, which does not precede it", l, h.kv_source_layer_index);
+                const uzu_layer_desc& src = desc->layers[h.kv_source_layer_index];
+                UZU_REQUIRE(src.mixer_kind == UZU_MIXER_LATENT_ATTENTION && !src.is_kv_sharing && src.latent_rank == h.latent_rank,
+                            "model_create: layer %u: the source layer %u must own latents of the same rank", l, h.kv_source_layer_index);
+            } else {
+                UZU_REQUIRE(full(h.latent_down, h.latent_rank, d) && h.latent_norm.present && h.latent_norm.scales, "model_create: layer %u owns its latents: down projection + latent norm required", l);
+            }
+        } else if (h.mixer_kind == UZU_MIXER_ATTENTION) {
+            UZU_REQUIRE(h.num_groups && h.num_heads % h.num_groups == 0, "model_create: layer %u: %u query heads on %u key / value heads", l, h.num_heads, h.num_groups);
+            UZU_UNSUPPORTED(h.has_gate || h.query_norm.present || h.key_norm.present || h.normalize_values || h.is_non_causal,
+                            "model_create: layer %u: gate / head norms / non-causal masks are options of the bf16-stream attention", l);
+            if (h.is_kv_sharing) {
+                UZU_REQUIRE(h.kv_source_layer_index < l, "model_create: layer %u shares the cache of layer %u, which does not precede it", l, h.kv_source_layer_index);
+                const uzu_layer_desc& src = desc->layers[h.kv_source_layer_index];
+                UZU_REQUIRE(src.mixer_kind == UZU_MIXER_ATTENTION && !src.is_kv_sharing && src.num_groups == h.num_groups && src.head_dim == h.head_dim && src.value_head_dim == h.value_head_dim,
+                            "model_create: layer %u: the source layer %u must own a cache of the same key / value heads and widths", l, h.kv_source_layer_index);
+                UZU_REQUIRE(full(h.qkv_projection, h.num_heads * h.head_dim, d), "model_create: layer %u reads another layer's cache: its projection yields queries only", l);
+            } else {
+                UZU_REQUIRE(full(h.qkv_projection, h.num_heads * h.head_dim + h.num_groups * (h.head_dim + h.value_head_dim), d),
+                            "model_create: layer %u: the packed projection must be a full-precision matrix [heads head_dim + groups (head_dim + value_head_dim), model_dim]", l);
+            }
         } else {
-            UZU_REQUIRE(full(h.latent_down, h.latent_rank, d) && h.latent_norm.present && h.latent_norm.scales, "model_create: layer %u owns its latents: down projection + latent norm required", l);
+            UZU_REQUIRE(full(h.qkv_projection, 2 * h.num_heads * h.head_dim + 2 * h.num_heads * h.value_head_dim, d) && !h.qkv_projection.out_biases,
+                        "model_create: layer %u: a retention layer's packed projection is queries | keys | values | gate without biases", l);
+            UZU_REQUIRE(h.retention_decay, "model_create: layer %u: retention without its decays", l);
+            UZU_UNSUPPORTED(!k::retention_supported(h.head_dim, h.value_head_dim), "model_create: layer %u: retention heads of %u x %u (keys up to 512, values up to 256)", l, h.head_dim,
+                            h.value_head_dim);
+            UZU_UNSUPPORTED(h.is_kv_sharing || h.sliding_window_size || h.has_sinks || h.unit_sink || h.score_soft_cap != 0.0f, "model_create: layer %u: attention options on a retention layer", l);
         }
         UZU_REQUIRE(!h.has_sinks || h.sinks, "model_create: layer %u: has_sinks without the tensor", l);
+        UZU_REQUIRE(!(h.has_sinks && h.unit_sink), "model_create: layer %u: sink logits and a unit sink exclude each other", l);
         UZU_REQUIRE(!h.depth_weights || h.num_depth_weights == l + 2, "model_create: layer %u: a depth mix takes %u weights", l, l + 2);
         if (!h.no_mlp) {
-            UZU_REQUIRE(h.pre_mlp_norm.present && h.pre_mlp_norm.kind == UZU_NORM_DYNAMIC_TANH && h.pre_mlp_norm.scales, "model_create: layer %u needs a dynamic-tanh pre-MLP norm", l);
+            UZU_REQUIRE(h.parallel_block ? !h.pre_mlp_norm.present : norm_ok(h.pre_mlp_norm), "model_create: layer %u: a pre-MLP norm (dynamic tanh or one-gain RMS), and none in a parallel block", l);
             if (h.mlp_kind == UZU_MLP_MOE) {
                 const uzu_moe_desc& M = h.moe;
-                UZU_REQUIRE(M.routing == UZU_MOE_ROUTE_SCORES && M.num_active_experts && M.num_active_experts <= M.num_routed_experts + M.num_identity_experts && M.router_weights &&
-                            (M.num_routed_experts == 0 || (M.expert_hidden_dim && M.w13 && M.w2)) && M.gating_sel == 2,
-                            "model_create: layer %u: score-routed SiLU-gated experts with their router and expert tensors", l);
+                UZU_REQUIRE((M.routing == UZU_MOE_ROUTE_SCORES || M.routing == UZU_MOE_ROUTE_TOPK_LOGITS) && M.num_active_experts &&
+                            M.num_active_experts <= M.num_routed_experts + M.num_identity_experts && M.router_weights &&
+                            (M.num_routed_experts == 0 || (M.expert_hidden_dim && M.w13 && M.w2)) && M.gating_sel == 2 && !M.up_biases && !M.down_biases,
+                            "model_create: layer %u: routed SiLU-gated experts without biases, with their router and expert tensors", l);
+                UZU_REQUIRE(M.routing == UZU_MOE_ROUTE_SCORES || (!M.num_identity_experts && !M.selection_bias), "model_create: layer %u: identity experts and selection biases belong to score routing", l);
             } else {
                 UZU_REQUIRE(h.mlp_plain && h.activation == UZU_ACT_RELU_SQUARED && full(h.up_projection, h.hidden_dim, d) && full(h.down_projection, d, h.hidden_dim),
                             "model_create: layer %u: the dense block is down(relu(up x + b)^2) + b with full-precision matrices", l);
@@ -384,6 +488,12 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
         X.alpha1 = h.pre_mixer_norm.alpha;
         TRY(upload_linear(m, h.qkv_projection, &L.qkv));
         TRY(upload_linear(m, h.out_projection, &L.out));
+        if (h.mixer_kind == UZU_MIXER_RETENTION) TRY(upload(m, h.retention_decay, (size_t)h.num_heads * 4, &X.decay));
+        if (h.unit_sink) { // a sink of logit 0 per head
+            std::vector<float> f(h.num_heads, 0.0f);
+            TRY(upload(m, f.data(), f.size() * 4, &X.sinks));
+        }
+        if (h.mixer_kind == UZU_MIXER_LATENT_ATTENTION) {
         TRY(upload_linear(m, h.latent_up_values, &L.lat_up_v));
         {   // W_up_k [heads * head_dim, rank] -> per head [rank, head_dim] (bf16 bits move, nothing is rounded)
             const uint32_t H = h.num_heads, hd = h.head_dim, rank = h.latent_rank;
@@ -398,6 +508,7 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
             TRY(upload_linear(m, h.latent_down, &L.lat_down));
             TRY(upload_norm(m, h.latent_norm, h.latent_rank, &L.lat_norm));
         }
+        } // latent attention
         if (h.has_sinks) {
             std::vector<float> f(h.num_heads);
             for (uint32_t i = 0; i < h.num_heads; ++i) f[i] = bf16_to_f32(((const uint16_t*)h.sinks)[i]);
@@ -406,12 +517,13 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
         if (h.token_shift) TRY(upload(m, h.token_shift, (size_t)d * 4, &X.token_shift));
         if (h.depth_weights) TRY(upload(m, h.depth_weights, (size_t)h.num_depth_weights * 4, &X.depth_weights));
         if (!h.no_mlp) {
-            TRY(upload_norm(m, h.pre_mlp_norm, d, &L.pre_mlp));
+            if (!h.parallel_block) TRY(upload_norm(m, h.pre_mlp_norm, d, &L.pre_mlp));
             X.alpha2 = h.pre_mlp_norm.alpha;
             if (h.mlp_kind == UZU_MLP_MOE) {
                 const uzu_moe_desc& M = h.moe;
                 const size_t E = M.num_routed_experts, ff = M.expert_hidden_dim;
                 TRY(upload(m, M.router_weights, (E + M.num_identity_experts) * d * 2, &L.moe.router_weights));
+                if (M.router_biases) TRY(upload(m, M.router_biases, (E + M.num_identity_experts) * 2, &L.moe.router_biases));
                 if (E) {
                     TRY(upload(m, M.w13, E * 2 * ff * d * 2, &L.moe.w13));
                     TRY(upload(m, M.w2, E * d * ff * 2, &L.moe.w2));
@@ -426,10 +538,36 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
                 w_hid = std::max(w_hid, h.hidden_dim);
             }
         }
-        w_q = std::max(w_q, h.num_heads * h.head_dim), w_rank = std::max(w_rank, h.latent_rank), w_lat = std::max(w_lat, h.num_heads * h.latent_rank);
+        w_q = std::max(w_q, h.qkv_projection.n), w_rank = std::max(w_rank, h.latent_rank), w_lat = std::max(w_lat, h.num_heads * h.latent_rank);
         w_attn = std::max(w_attn, h.num_heads * h.value_head_dim);
     }
+    if (!desc->tied_embeddings) TRY(upload_linear(m, desc->output_embedding, &m->output_embedding));
+    {   // one table pair per distinct rotation; a layer points at its own
+        const uint32_t n_ropes = desc->num_ropes ? desc->num_ropes : (desc->rope.kind != UZU_ROPE_NONE ? 1u : 0u);
+        m->ropes.resize(n_ropes);
+        const size_t saved = m->weight_bytes;
+        for (uint32_t r = 0; r < n_ropes; ++r) {
+            const uzu_rope_desc& Rd = desc->num_ropes ? desc->ropes[r] : desc->rope;
+            if (Rd.kind == UZU_ROPE_NONE || !Rd.head_dim) {
+                set_error("model_create: RoPE configuration %u is empty", r);
+                return fail(UZU_ERR_INVALID_ARGUMENT);
+            }
+            std::vector<float> c, sn;
+            rope_tables(Rd, m->max_positions, c, sn);
+            TRY(upload(m, c.data(), c.size() * 4, &m->ropes[r].cos));
+            TRY(upload(m, sn.data(), sn.size() * 4, &m->ropes[r].sin));
+            m->ropes[r].dim = Rd.head_dim;
+        }
+        m->weight_bytes = saved;
+        for (DLayer& L : m->layers)
+            if (L.d.use_rope) {
+                const uzu_hip_model::RopeTable& T = m->ropes[desc->num_ropes ? L.d.rope_index : 0];
+                L.rope_cos = T.cos, L.rope_sin = T.sin, L.rope_dim = T.dim;
+            }
+    }
     const size_t R = S.max_rows;
+    if (!w_lat) w_lat = 1;
+    if (!w_rank) w_rank = 1;
     TRY(need_f32(m, (size_t)(nl + 1) * R * d, &S.slots));
     TRY(need_f32(m, R * d, &S.xin));
     TRY(need_f32(m, R * d, &S.normed));
@@ -456,6 +594,7 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
     TRY(dev_alloc(m, R * 4, &p)); S.d_row_seq = (uint32_t*)p;
     TRY(dev_alloc(m, R * 4, &p)); S.d_out_rows = (uint32_t*)p;
     TRY(dev_alloc(m, (size_t)nl * S.max_seqs * sizeof(void*), &p)); S.d_cache_ptrs = (void**)p;
+    TRY(dev_alloc(m, (size_t)nl * S.max_seqs * sizeof(void*), &p)); S.d_cache2_ptrs = (void**)p;
     TRY(dev_alloc(m, (size_t)nl * S.max_seqs * sizeof(float*), &p)); S.d_shift_ptrs = (float**)p;
     TRY(dev_alloc(m, R * 4, &p)); m->batch_tokens = (uint32_t*)p;
     if (flags & UZU_MODEL_DEBUG_TAPS) TRY(need_f32(m, (size_t)nl * R * d, &S.taps));
@@ -493,9 +632,20 @@ void s32_destroy(uzu_hip_model* m) {
 uzu_status s32_state_layer(uzu_hip_model* m, uzu_hip_state* st, uint32_t l) {
     const uzu_layer_desc& h = m->layers[l].d;
     void* p = nullptr;
-    if (!h.is_kv_sharing) { // rows are written before they are read (latent_norm_append precedes the core in every pass)
-        UZU_PROPAGATE(state_alloc(st, (size_t)m->max_positions * h.latent_rank * (m->s32->full_f32 ? 4 : 2), &p, false));
-        st->layers[l].latent = p;
+    const size_t elem = m->s32->full_f32 ? 4 : 2;
+    if (h.mixer_kind == UZU_MIXER_RETENTION) { // read only behind position 0, where the kernel starts from zeros: no fill needed
+        UZU_PROPAGATE(state_alloc(st, (size_t)h.num_heads * h.head_dim * h.value_head_dim * 4, &p, false));
+        st->layers[l].ret_state = (float*)p;
+    } else if (!h.is_kv_sharing) { // rows are written before they are read (the append precedes the core in every pass)
+        if (h.mixer_kind == UZU_MIXER_ATTENTION) {
+            UZU_PROPAGATE(state_alloc(st, (size_t)m->max_positions * h.num_groups * h.head_dim * elem, &p, false));
+            st->layers[l].cache_k = p;
+            UZU_PROPAGATE(state_alloc(st, (size_t)m->max_positions * h.num_groups * h.value_head_dim * elem, &p, false));
+            st->layers[l].cache_v = p;
+        } else {
+            UZU_PROPAGATE(state_alloc(st, (size_t)m->max_positions * h.latent_rank * elem, &p, false));
+            st->layers[l].latent = p;
+        }
     }
     if (h.token_shift) {
         UZU_PROPAGATE(state_alloc(st, (size_t)m->d.model_dim * 4, &p));

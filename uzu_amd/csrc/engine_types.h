@@ -122,6 +122,10 @@ struct uzu_hip_state {
         // f32-stream designs: the latent cache of a layer that owns one ([max positions][latent_rank], bf16 or f32) and the token shift's last normalised row
         void* latent = nullptr;
         float* shift_prev = nullptr;
+        // ... an attention layer that owns its cache: rotated keys [max positions][groups * head_dim] and values [max positions][groups * value_head_dim]
+        // (bf16 or f32); a retention layer: the f32 state [heads][head_dim][value_head_dim]
+        void *cache_k = nullptr, *cache_v = nullptr;
+        float* ret_state = nullptr;
     };
     std::vector<Layer> layers;
     uint32_t *d_ctx_len = nullptr, *d_tokens = nullptr, *d_out_token = nullptr, *d_sampled = nullptr;

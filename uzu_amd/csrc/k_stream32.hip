@@ -37,13 +37,34 @@ __device__ __forceinline__ float lane_dot(const float* x, const uint16_t* w, uin
     return acc;
 }
 
-__global__ void __launch_bounds__(256) embed_rows_f32_kernel(const uint32_t* tokens, const uint16_t* table, float* out, uint32_t vocab, uint32_t d) {
+__global__ void __launch_bounds__(256) embed_rows_f32_kernel(const uint32_t* tokens, const uint16_t* table, float* out, uint32_t vocab, uint32_t d, float scale) {
     const uint32_t r = blockIdx.x;
     uint32_t t = tokens[r];
     if (t >= vocab) t = 0;
     const uint16_t* src = table + (size_t)t * d;
     float* dst = out + (size_t)r * d;
-    for (uint32_t i = threadIdx.x; i < d; i += blockDim.x) dst[i] = bf16_to_f32(src[i]);
+    for (uint32_t i = threadIdx.x; i < d; i += blockDim.x) dst[i] = bf16_to_f32(src[i]) * scale; // (scale 1: the value itself)
+}
+
+// a workgroup per row: the sum of squares as 256 strided partial sums folded in a fixed tree, then the scaled row
+__global__ void __launch_bounds__(256) rms_norm_rows_kernel(const float* x, float* out, const float* scales, float gain, float eps, const uint32_t* row_index, uint32_t d) {
+    __shared__ float s_red[256];
+    const uint32_t r = blockIdx.x;
+    const float* xr = x + (size_t)(row_index ? row_index[r] : r) * d;
+    float acc = 0.0f;
+    for (uint32_t i = threadIdx.x; i < d; i += 256) acc = fmaf(xr[i], xr[i], acc);
+    s_red[threadIdx.x] = acc;
+    __syncthreads();
+    for (uint32_t w = 128; w > 0; w >>= 1) {
+        if (threadIdx.x < w) s_red[threadIdx.x] += s_red[threadIdx.x + w];
+        __syncthreads();
+    }
+    const float inv = 1.0f / sqrtf(s_red[0] / (float)d + eps);
+    float* o = out + (size_t)r * d;
+    for (uint32_t i = threadIdx.x; i < d; i += 256) {
+        const float v = xr[i] * inv * gain;
+        o[i] = scales ? v * scales[i] : v;
+    }
 }
 
 __global__ void __launch_bounds__(256) dyn_tanh_kernel(DynTanhParams p) {
@@ -82,6 +103,11 @@ __global__ void __launch_bounds__(256) depth_mix_kernel(const float* slots, size
     float acc = 0.0f;
     for (uint32_t j = 0; j < count; ++j) acc = fmaf(w[j], slots[(size_t)j * slot_stride + i], acc);
     out[i] = acc;
+}
+
+__device__ __forceinline__ float expert_act(float gate, float up, const ExpertAct& a) {
+    const float g = fminf(fmaxf(gate, a.gate_min), a.gate_max), u = fminf(fmaxf(up, a.up_min), a.up_max);
+    return g / (1.0f + expf(-(a.alpha * g))) * (u + a.up_offset);
 }
 
 __device__ __forceinline__ float apply_act(float v, uint32_t act) {
@@ -204,8 +230,10 @@ __global__ void __launch_bounds__(256) linear_tile_kernel(LinearF32Params p) {
 
 // ---- score routing: one wave per row
 constexpr uint32_t kRouteMaxOutputs = 512; // 8 per lane
+// mode 0: score routing (softmax over all outputs, choice by score + selection_bias, weights = winners' scores / their sum)
+// mode 1 / 2: top-k of the logits z + router_bias; weights = the winners' logits (1) or the softmax over them (2)
 __global__ void __launch_bounds__(64) moe_route_scores_kernel(const float* x, const uint16_t* router, const float* selection_bias, int32_t* ids, float* weights, uint32_t d,
-                                                              uint32_t outputs, uint32_t top) {
+                                                              uint32_t outputs, uint32_t top, uint32_t mode, const uint16_t* router_bias) {
     const uint32_t r = blockIdx.x, lane = threadIdx.x;
     const float* xr = x + (size_t)r * d;
     float z[8];
@@ -214,6 +242,7 @@ __global__ void __launch_bounds__(64) moe_route_scores_kernel(const float* x, co
     for (int j = 0; j < 8; ++j) z[j] = -INFINITY;
     for (uint32_t e = 0; e < outputs; ++e) {
         float acc = wave_sum(lane_dot(xr, router + (size_t)e * d, d, lane));
+        if (router_bias) acc += bf16_to_f32(router_bias[e]);
         if ((e & 63) == lane) {
 #pragma unroll
             for (int j = 0; j < 8; ++j)
@@ -233,9 +262,10 @@ __global__ void __launch_bounds__(64) moe_route_scores_kernel(const float* x, co
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
         const uint32_t e = j * 64 + lane;
-        score[j] = ex[j] / sum;
+        score[j] = mode ? z[j] : ex[j] / sum;
         choice[j] = e < outputs ? score[j] + (selection_bias ? selection_bias[e] : 0.0f) : -INFINITY;
     }
+    float first = 0.0f; // the largest winner (mode 2: the softmax's reference point)
     float wsum = 0.0f;
     float my_w = 0.0f; // lane t keeps the t-th winner's score
     int32_t my_id = 0;
@@ -257,6 +287,8 @@ __global__ void __launch_bounds__(64) moe_route_scores_kernel(const float* x, co
 #pragma unroll
         for (int j = 0; j < 8; ++j)
             if ((uint32_t)j * 64 + lane == best_e) choice[j] = -INFINITY; // taken (a NaN row leaves best_e invalid: every lane then agrees on 0xFFFFFFFF)
+        if (t == 0) first = best_s;
+        if (mode == 2) best_s = expf(best_s - first);
         wsum += best_s;
         if ((t & 63) == lane && t < 64) my_w = best_s, my_id = (int32_t)best_e;
         if (t >= 64 && lane == 0) { // more winners than lanes: written as they come
@@ -266,13 +298,13 @@ __global__ void __launch_bounds__(64) moe_route_scores_kernel(const float* x, co
     }
     if (lane < top && lane < 64) {
         ids[(size_t)r * top + lane] = my_id;
-        weights[(size_t)r * top + lane] = my_w / (wsum + 1e-20f);
+        weights[(size_t)r * top + lane] = mode == 1 ? my_w : mode == 2 ? my_w / wsum : my_w / (wsum + 1e-20f);
     }
 }
 
 // a workgroup per (row, slot): the row once into LDS, then a wave per hidden unit (gate and up rows of the unit in the same pass)
 __global__ void __launch_bounds__(256) moe_experts_gate_up_kernel(const float* x, const int32_t* ids, const uint16_t* w13, float* hidden, uint32_t d, uint32_t ff, uint32_t routed,
-                                                                  uint32_t top, uint32_t bf16_products) {
+                                                                  uint32_t top, uint32_t bf16_products, ExpertAct act) {
     extern __shared__ float s_x[];
     const uint32_t slot = blockIdx.x, r = slot / top;
     const int32_t e = ids[slot];
@@ -285,7 +317,7 @@ __global__ void __launch_bounds__(256) moe_experts_gate_up_kernel(const float* x
         const uint16_t* wu = base + (size_t)f * d;
         const uint16_t* wg = base + (size_t)(ff + f) * d;
         const float au = wave_sum(lane_dot(s_x, wu, d, lane)), ag = wave_sum(lane_dot(s_x, wg, d, lane));
-        if (lane == 0) hidden[(size_t)slot * ff + f] = ag / (1.0f + expf(-ag)) * au;
+        if (lane == 0) hidden[(size_t)slot * ff + f] = expert_act(ag, au, act);
     }
 }
 
@@ -354,13 +386,13 @@ __global__ void __launch_bounds__(256) moe_scatter_kernel(const int32_t* ids, ui
     perm[pos] = i / top;
     slot_pos[i] = pos;
 }
-__global__ void __launch_bounds__(256) moe_act_mul_kernel(const float* y1, float* hidden, const uint32_t* offsets, uint32_t routed, uint32_t ff) {
+__global__ void __launch_bounds__(256) moe_act_mul_kernel(const float* y1, float* hidden, const uint32_t* offsets, uint32_t routed, uint32_t ff, ExpertAct act) {
     const uint32_t pos = blockIdx.x;
     if (pos >= offsets[routed]) return;
     const float* src = y1 + (size_t)pos * 2 * ff;
     for (uint32_t f = threadIdx.x; f < ff; f += blockDim.x) {
         const float g = src[ff + f];
-        hidden[(size_t)pos * ff + f] = g / (1.0f + expf(-g)) * src[f];
+        hidden[(size_t)pos * ff + f] = expert_act(g, src[f], act);
     }
 }
 __global__ void __launch_bounds__(256) moe_combine_kernel(const float* y2, const float* x, const int32_t* ids, const float* weights, const uint32_t* slot_pos, const float* residual,
@@ -400,7 +432,7 @@ uzu_status moe_experts_grouped(hipStream_t s, const MoeGroupedParams& p) {
     q.x = p.x, q.w = p.w13, q.y = p.y1, q.rows = slots, q.n = 2 * p.ff, q.k = p.d, q.ldx = p.d, q.ldy = 2 * p.ff, q.batch = p.routed, q.w_batch = (size_t)2 * p.ff * p.d;
     q.bf16_products = 1, q.row_offsets = p.offsets, q.row_map = p.perm;
     UZU_PROPAGATE(linear_mfma(s, q));
-    UZU_PROPAGATE(launch_check([&] { hipLaunchKernelGGL(moe_act_mul_kernel, dim3(slots), dim3(256), 0, s, p.y1, p.hidden, p.offsets, p.routed, p.ff); }, "moe_act_mul"));
+    UZU_PROPAGATE(launch_check([&] { hipLaunchKernelGGL(moe_act_mul_kernel, dim3(slots), dim3(256), 0, s, p.y1, p.hidden, p.offsets, p.routed, p.ff, p.act); }, "moe_act_mul"));
     LinearF32Params r{};
     r.x = p.hidden, r.w = p.w2, r.y = p.y2, r.rows = slots, r.n = p.d, r.k = p.ff, r.ldx = p.ff, r.ldy = p.d, r.batch = p.routed, r.w_batch = (size_t)p.d * p.ff;
     r.bf16_products = 1, r.row_offsets = p.offsets;
@@ -409,9 +441,15 @@ uzu_status moe_experts_grouped(hipStream_t s, const MoeGroupedParams& p) {
                         "moe_combine");
 }
 
-uzu_status embed_rows_f32(hipStream_t s, const uint32_t* tokens, const uint16_t* table, float* out, uint32_t rows, uint32_t vocab, uint32_t d) {
+uzu_status embed_rows_f32(hipStream_t s, const uint32_t* tokens, const uint16_t* table, float* out, uint32_t rows, uint32_t vocab, uint32_t d, float scale) {
     if (!rows) return UZU_OK;
-    return launch_check([&] { hipLaunchKernelGGL(embed_rows_f32_kernel, dim3(rows), dim3(256), 0, s, tokens, table, out, vocab, d); }, "embed_rows_f32");
+    return launch_check([&] { hipLaunchKernelGGL(embed_rows_f32_kernel, dim3(rows), dim3(256), 0, s, tokens, table, out, vocab, d, scale); }, "embed_rows_f32");
+}
+
+uzu_status rms_norm_rows(hipStream_t s, const float* x, float* out, const float* scales, float gain, float eps, const uint32_t* row_index, uint32_t rows, uint32_t d) {
+    if (!rows) return UZU_OK;
+    UZU_REQUIRE(x && out && d, "rms_norm_rows: null argument");
+    return launch_check([&] { hipLaunchKernelGGL(rms_norm_rows_kernel, dim3(rows), dim3(256), 0, s, x, out, scales, gain, eps, row_index, d); }, "rms_norm_rows");
 }
 
 uzu_status dyn_tanh_norm(hipStream_t s, const DynTanhParams& p) {
@@ -465,17 +503,25 @@ uzu_status moe_route_scores(hipStream_t s, const float* x, const uint16_t* route
                             uint32_t outputs, uint32_t top) {
     if (!rows) return UZU_OK;
     UZU_UNSUPPORTED(outputs > kRouteMaxOutputs || top > 64 || top > outputs || !top, "moe_route_scores: at most %u router outputs and 64 winners (got %u, %u)", kRouteMaxOutputs, outputs, top);
-    return launch_check([&] { hipLaunchKernelGGL(moe_route_scores_kernel, dim3(rows), dim3(64), 0, s, x, router, selection_bias, ids, weights, d, outputs, top); }, "moe_route_scores");
+    return launch_check([&] { hipLaunchKernelGGL(moe_route_scores_kernel, dim3(rows), dim3(64), 0, s, x, router, selection_bias, ids, weights, d, outputs, top, 0u, (const uint16_t*)nullptr); }, "moe_route_scores");
+}
+
+uzu_status moe_route_topk(hipStream_t s, const float* x, const uint16_t* router, const uint16_t* router_bias, int32_t* ids, float* weights, uint32_t rows, uint32_t d,
+                          uint32_t outputs, uint32_t top, uint32_t renorm) {
+    if (!rows) return UZU_OK;
+    UZU_UNSUPPORTED(outputs > kRouteMaxOutputs || top > 64 || top > outputs || !top, "moe_route_topk: at most %u router outputs and 64 winners (got %u, %u)", kRouteMaxOutputs, outputs, top);
+    return launch_check([&] { hipLaunchKernelGGL(moe_route_scores_kernel, dim3(rows), dim3(64), 0, s, x, router, (const float*)nullptr, ids, weights, d, outputs, top, renorm ? 2u : 1u, router_bias); },
+                        "moe_route_topk");
 }
 
 uzu_status moe_experts_gate_up(hipStream_t s, const float* x, const int32_t* ids, const uint16_t* w13, float* hidden, uint32_t rows, uint32_t d, uint32_t ff, uint32_t routed,
-                               uint32_t top, uint32_t bf16_products) {
+                               uint32_t top, uint32_t bf16_products, const ExpertAct& act) {
     if (!rows || !routed) return UZU_OK;
     UZU_UNSUPPORTED((size_t)d * 4 > 48 * 1024, "moe_experts_gate_up: model_dim %u does not fit the workgroup's LDS row", d);
     // few (row, slot) pairs (decode): the hidden units of a pair are spread over more workgroups, so that the expert's rows stream through many CUs
     const uint32_t want = (1024 + rows * top - 1) / (rows * top), most = (ff + 15) / 16;
     const uint32_t gy = want < 1 ? 1 : (want > most ? most : want);
-    return launch_check([&] { hipLaunchKernelGGL(moe_experts_gate_up_kernel, dim3(rows * top, gy), dim3(256), (size_t)d * 4, s, x, ids, w13, hidden, d, ff, routed, top, bf16_products); },
+    return launch_check([&] { hipLaunchKernelGGL(moe_experts_gate_up_kernel, dim3(rows * top, gy), dim3(256), (size_t)d * 4, s, x, ids, w13, hidden, d, ff, routed, top, bf16_products, act); },
                         "moe_experts_gate_up");
 }
 

@@ -1,0 +1,168 @@
+// k_window_attention.hip -- attention over a per-position cache of rotated keys and values for the f32-stream designs (kernels_stream32.h): rotation + key
+// scaling + cache append, and the attention core with grouped heads, a soft cap on the scores, a causal sliding window and sink terms in the softmax denominator.
+//
+// Scores, softmax weights and the weighted sums are f32 whatever the cache holds (bf16 rows in the serving precision, f32 rows in the full-f32 mode).  A row's
+// keys are walked in blocks of 64 counted from the first key the row sees, so the order of every sum depends on the row's position and the window only: not on
+// how a prompt was cut into passes, and not on what else a pass carries.
+#include "device_utils.h"
+#include "kernels_stream32.h"
+
+namespace uzu {
+namespace k {
+
+namespace {
+
+__device__ __forceinline__ float cache_ld(const void* p, uint32_t is_bf16, size_t i) { return is_bf16 ? bf16_to_f32(((const uint16_t*)p)[i]) : ((const float*)p)[i]; }
+__device__ __forceinline__ void cache_st(void* p, uint32_t is_bf16, size_t i, float v) {
+    if (is_bf16) ((uint16_t*)p)[i] = f32_to_bf16(v);
+    else ((float*)p)[i] = v;
+}
+
+// a workgroup per row: query pairs in place, key pairs (+ the unrotated tail) to the cache or in place, values to the cache
+__global__ void __launch_bounds__(256) rope_append_kernel(RopeAppendParams p) {
+    const uint32_t r = blockIdx.x;
+    const uint32_t z = p.row_seq[r];
+    const SeqSpan sp = p.spans[z];
+    const uint32_t t = sp.start + (r - sp.row0);
+    float* row = p.qkv + (size_t)r * p.ld;
+    const uint32_t half = p.rope_dim / 2;
+    const float* cs = p.cosines + (size_t)t * p.rope_dim;
+    const float* sn = p.sines + (size_t)t * p.rope_dim;
+    for (uint32_t idx = threadIdx.x; idx < p.heads * half; idx += 256) {
+        const uint32_t a = idx / half, i = idx - a * half;
+        float* h = row + (size_t)a * p.dim;
+        const float u = h[i], v = h[i + half], c = cs[i], s = sn[i];
+        h[i] = u * c - v * s;
+        h[i + half] = v * c + u * s;
+    }
+    if (!p.kv_heads) return;
+    const float ks = p.key_scale;
+    void* kc = p.key_caches ? p.key_caches[z] : nullptr;
+    const size_t krow = (size_t)t * p.kv_heads * p.dim;
+    for (uint32_t idx = threadIdx.x; idx < p.kv_heads * p.dim; idx += 256) {
+        const uint32_t g = idx / p.dim, c = idx - g * p.dim;
+        float* h = row + p.k_col + (size_t)g * p.dim;
+        if (c < half) {
+            const float u = h[c], v = h[c + half], co = cs[c], s = sn[c];
+            const float a = (u * co - v * s) * ks, b = (v * co + u * s) * ks;
+            if (kc) cache_st(kc, p.cache_bf16, krow + idx, a), cache_st(kc, p.cache_bf16, krow + idx + half, b);
+            else h[c] = a, h[c + half] = b;
+        } else if (c >= p.rope_dim) {
+            const float a = h[c] * ks;
+            if (kc) cache_st(kc, p.cache_bf16, krow + idx, a);
+            else h[c] = a;
+        }
+    }
+    if (p.value_caches) {
+        void* vc = p.value_caches[z];
+        const size_t vrow = (size_t)t * p.kv_heads * p.vdim;
+        for (uint32_t idx = threadIdx.x; idx < p.kv_heads * p.vdim; idx += 256) cache_st(vc, p.cache_bf16, vrow + idx, row[p.v_col + idx]);
+    }
+}
+
+// ---- the simple form: a wave per (row, head).  Keys in blocks of 64 from the row's first visible key: a lane scores one key of the block (the whole dot
+// product, the query staged in LDS), the block's weights go through LDS, then a lane owns value coordinates lane, lane + 64, ... of the running sum.
+constexpr uint32_t kMaxVecPerLane = 8; // value widths up to 512
+__global__ void __launch_bounds__(64) window_attention_simple_kernel(WindowAttentionParams p) {
+    extern __shared__ float s_mem[]; // [dim] query + [64] weights
+    float* s_q = s_mem;
+    float* s_p = s_mem + p.dim;
+    const uint32_t r = blockIdx.x, a = blockIdx.y, lane = threadIdx.x;
+    const uint32_t z = p.row_seq[r];
+    const SeqSpan sp = p.spans[z];
+    const uint32_t t = sp.start + (r - sp.row0);
+    const uint32_t g = a / (p.heads / p.kv_heads);
+    const void* K = p.key_caches[z];
+    const void* V = p.value_caches[z];
+    const uint32_t lo = (p.window && t + 1 > p.window) ? t + 1 - p.window : 0u;
+    const float* q = p.q + (size_t)r * p.ldq + (size_t)a * p.dim;
+    for (uint32_t c = lane; c < p.dim; c += 64) s_q[c] = q[c];
+    __syncthreads();
+    float m = p.sinks ? p.sinks[a] : -INFINITY, l = p.sinks ? 1.0f : 0.0f;
+    float acc[kMaxVecPerLane];
+#pragma unroll
+    for (uint32_t i = 0; i < kMaxVecPerLane; ++i) acc[i] = 0.0f;
+    const size_t kpitch = (size_t)p.kv_heads * p.dim, vpitch = (size_t)p.kv_heads * p.vdim;
+    for (uint32_t j0 = lo; j0 <= t; j0 += 64) {
+        const uint32_t j = j0 + lane;
+        float s = -INFINITY;
+        if (j <= t) {
+            const size_t base = (size_t)j * kpitch + (size_t)g * p.dim;
+            float dot = 0.0f;
+            if (p.cache_bf16) {
+                const uint16_t* kr = (const uint16_t*)K + base;
+                if ((p.dim & 7) == 0 && (((uintptr_t)kr) & 15) == 0) {
+                    for (uint32_t c = 0; c < p.dim; c += 8) {
+                        const uint4 kv = *(const uint4*)(kr + c);
+                        const uint32_t w[4] = {kv.x, kv.y, kv.z, kv.w};
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            dot = fmaf(s_q[c + 2 * i], bits_to_f32(w[i] << 16), dot);
+                            dot = fmaf(s_q[c + 2 * i + 1], bits_to_f32(w[i] & 0xFFFF0000u), dot);
+                        }
+                    }
+                } else {
+                    for (uint32_t c = 0; c < p.dim; ++c) dot = fmaf(s_q[c], bf16_to_f32(kr[c]), dot);
+                }
+            } else {
+                const float* kr = (const float*)K + base;
+                for (uint32_t c = 0; c < p.dim; ++c) dot = fmaf(s_q[c], kr[c], dot);
+            }
+            s = dot * p.scale;
+            if (p.soft_cap != 0.0f) s = p.soft_cap * tanhf(s / p.soft_cap);
+        }
+        const float m_new = fmaxf(m, wave_max(s));
+        const float w = j <= t ? expf(s - m_new) : 0.0f;
+        const float corr = expf(m - m_new); // (first block without a sink: exp(-inf) = 0 against l = 0 and zero sums)
+        l = l * corr + wave_sum(w);
+        m = m_new;
+        __syncthreads();
+        s_p[lane] = w;
+        __syncthreads();
+        const uint32_t nk = t - j0 + 1 < 64 ? t - j0 + 1 : 64;
+#pragma unroll
+        for (uint32_t i = 0; i < kMaxVecPerLane; ++i) {
+            const uint32_t c = lane + 64 * i;
+            if (c >= p.vdim) break;
+            float sum = acc[i] * corr;
+            const size_t vb = (size_t)j0 * vpitch + (size_t)g * p.vdim + c;
+            for (uint32_t jj = 0; jj < nk; ++jj) sum = fmaf(s_p[jj], cache_ld(V, p.cache_bf16, vb + (size_t)jj * vpitch), sum);
+            acc[i] = sum;
+        }
+    }
+    float* o = p.out + ((size_t)r * p.heads + a) * p.vdim;
+#pragma unroll
+    for (uint32_t i = 0; i < kMaxVecPerLane; ++i) {
+        const uint32_t c = lane + 64 * i;
+        if (c >= p.vdim) break;
+        o[c] = acc[i] / l;
+    }
+}
+
+} // namespace
+
+uzu_status rope_append(hipStream_t s, const RopeAppendParams& p) {
+    if (!p.rows) return UZU_OK;
+    UZU_REQUIRE(p.qkv && p.spans && p.row_seq && p.heads && p.dim, "rope_append: null argument");
+    UZU_REQUIRE(p.rope_dim % 2 == 0 && p.rope_dim <= p.dim && (!p.rope_dim || (p.cosines && p.sines)), "rope_append: rotation width %u of a head of %u (even, with its tables)", p.rope_dim, p.dim);
+    UZU_REQUIRE(!p.kv_heads || ((p.key_caches != nullptr) == (p.value_caches != nullptr)), "rope_append: key and value caches come together");
+    return launch_check([&] { hipLaunchKernelGGL(rope_append_kernel, dim3(p.rows), dim3(256), 0, s, p); }, "rope_append");
+}
+
+uzu_status window_attention_mfma(hipStream_t s, const WindowAttentionParams& p); // k_window_attention_mfma.hip
+
+uzu_status window_attention(hipStream_t s, const WindowAttentionParams& p) {
+    if (!p.rows) return UZU_OK;
+    UZU_REQUIRE(p.q && p.out && p.key_caches && p.value_caches && p.spans && p.row_seq, "window_attention: null argument");
+    UZU_REQUIRE(p.heads && p.kv_heads && p.heads % p.kv_heads == 0 && p.dim && p.vdim, "window_attention: %u query heads on %u key / value heads", p.heads, p.kv_heads);
+    UZU_UNSUPPORTED(p.vdim > 64 * kMaxVecPerLane || p.dim > 8192, "window_attention: value width %u (at most %u)", p.vdim, 64 * kMaxVecPerLane);
+    if (p.form == 2 || (p.form == 0 && window_attention_mfma_supported(p))) {
+        UZU_UNSUPPORTED(!window_attention_mfma_supported(p), "window_attention: the matrix-core form does not take this shape");
+        return window_attention_mfma(s, p);
+    }
+    UZU_REQUIRE(p.heads <= 65535, "window_attention: too many heads for one launch");
+    return launch_check([&] { hipLaunchKernelGGL(window_attention_simple_kernel, dim3(p.rows, p.heads), dim3(64), (size_t)(p.dim + 64) * 4, s, p); }, "window_attention");
+}
+
+} // namespace k
+} // namespace uzu

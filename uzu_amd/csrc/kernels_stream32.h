@@ -4,6 +4,8 @@
 //   k_stream32.hip           embedding rows, dynamic-tanh norm + token shift, depth mix, the full-precision linear, score-routed experts
 //   k_linear_mfma.hip        the full-precision linear on the matrix cores (bf16 products, prefill-sized row counts)
 //   k_latent_attention.hip   latent normalisation + cache append, the latent-space attention core (prompt rows and decode rows)
+//   k_window_attention.hip   rotation + key / value cache append, attention over cached keys and values (grouped heads, score cap, window, sinks)
+//   k_retention.hip          retention: the decayed outer-product state (token by token and in chunks), per-head RMS division + gate
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -19,8 +21,12 @@ struct SeqSpan {
     uint32_t row0, count, start;
 };
 
-// out[r, :] = f32(table[token[r], :])   (table bf16 [vocab, d]; an id >= vocab reads row 0 and the host has refused it before)
-uzu_status embed_rows_f32(hipStream_t s, const uint32_t* tokens, const uint16_t* table, float* out, uint32_t rows, uint32_t vocab, uint32_t d);
+// out[r, :] = f32(table[token[r], :]) * scale   (table bf16 [vocab, d]; an id >= vocab reads row 0 and the host has refused it before)
+uzu_status embed_rows_f32(hipStream_t s, const uint32_t* tokens, const uint16_t* table, float* out, uint32_t rows, uint32_t vocab, uint32_t d, float scale = 1.0f);
+
+// RMS norm with one gain: out[r, :] = gain * x[src(r), :] / sqrt(mean(x[src(r), :]^2) + eps),   src(r) = row_index ? row_index[r] : r.
+// scales (f32 [d], optional) multiplies per coordinate on top.  The row's sum of squares is taken in a fixed order.
+uzu_status rms_norm_rows(hipStream_t s, const float* x, float* out, const float* scales, float gain, float eps, const uint32_t* row_index, uint32_t rows, uint32_t d);
 
 // Dynamic-tanh norm, optionally followed by the token shift:
 //   h[r]   = tanh(alpha * x[src(r)]) * scales + biases          src(r) = row_index ? row_index[r] : r
@@ -76,9 +82,18 @@ size_t linear_f32_bytes(const LinearF32Params& p);
 // weights = score / (sum of the winners' scores + 1e-20).  ids [rows, top] (>= routed: an identity expert), weights f32 [rows, top].
 uzu_status moe_route_scores(hipStream_t s, const float* x, const uint16_t* router, const float* selection_bias, int32_t* ids, float* weights, uint32_t rows, uint32_t d,
                             uint32_t outputs, uint32_t top);
-// hidden[r * top + j, f] = silu(gate_e x_r) * (up_e x_r) for e = ids[r, j] < routed; w13 bf16 [routed][2 ff][d], rows [0, ff) of an expert = up, [ff, 2 ff) = gate
+// Top-k routing: per row logits z = router x + bias (f32; bias bf16 [outputs] or null), the `top` largest win (ties: lower index); weights = softmax over the
+// winners' logits (renorm != 0) or the logits themselves.  ids / weights [rows, top], winners by falling logit.
+uzu_status moe_route_topk(hipStream_t s, const float* x, const uint16_t* router, const uint16_t* router_bias, int32_t* ids, float* weights, uint32_t rows, uint32_t d,
+                          uint32_t outputs, uint32_t top, uint32_t renorm);
+// The gated product of an expert's hidden unit: g = clamp(gate, gate_min, gate_max), u = clamp(up, up_min, up_max), g * sigmoid(alpha * g) * (u + up_offset).
+// The default is silu(gate) * up.
+struct ExpertAct {
+    float alpha = 1.0f, gate_min = -INFINITY, gate_max = INFINITY, up_min = -INFINITY, up_max = INFINITY, up_offset = 0.0f;
+};
+// hidden[r * top + j, f] = act(gate_e x_r, up_e x_r) for e = ids[r, j] < routed; w13 bf16 [routed][2 ff][d], rows [0, ff) of an expert = up, [ff, 2 ff) = gate
 uzu_status moe_experts_gate_up(hipStream_t s, const float* x, const int32_t* ids, const uint16_t* w13, float* hidden, uint32_t rows, uint32_t d, uint32_t ff, uint32_t routed,
-                               uint32_t top, uint32_t bf16_products);
+                               uint32_t top, uint32_t bf16_products, const ExpertAct& act = ExpertAct());
 // y[r, :] = residual[r, :] + sum_j weights[r, j] * (ids[r, j] < routed ? down_e hidden[r * top + j] : x[r, :])   in slot order; w2 bf16 [routed][d][ff]; y may alias residual
 uzu_status moe_experts_down_combine(hipStream_t s, const float* hidden, const float* x, const int32_t* ids, const float* weights, const uint16_t* w2, const float* residual,
                                     float* y, uint32_t rows, uint32_t d, uint32_t ff, uint32_t routed, uint32_t top, uint32_t bf16_products);
@@ -96,6 +111,7 @@ struct MoeGroupedParams {
     float *y1, *hidden, *y2;
     uint32_t *perm, *slot_pos, *offsets, *cursor;
     uint32_t rows, d, ff, routed, top;
+    ExpertAct act;
 };
 bool moe_experts_grouped_supported(const MoeGroupedParams& p);
 uzu_status moe_experts_grouped(hipStream_t s, const MoeGroupedParams& p);
@@ -131,6 +147,73 @@ size_t latent_attention_split_ws_bytes(uint32_t rows, uint32_t heads, uint32_t r
 bool latent_attention_tiled_supported(const LatentAttentionParams& p);
 uzu_status latent_attention(hipStream_t s, const LatentAttentionParams& p);
 constexpr uint32_t kLatentMaxRank = 2048;
+
+// Rotation of queries and keys, key scaling, and the append of keys and values to the sequences' caches -- what stands between the packed projection and the
+// mixer's core.  Row r of `qkv` (f32, pitch ld) holds queries [heads][dim] at column 0, keys [kv_heads][dim] at column k_col and values [kv_heads][vdim] at
+// column v_col.  The first rope_dim coordinates of every query and key head turn by the angle of the row's position t: with half = rope_dim / 2,
+//   (a_i, a_(i+half)) <- (a_i cos[t, i] - a_(i+half) sin[t, i], a_(i+half) cos[t, i] + a_i sin[t, i])      (tables f32 [positions][rope_dim])
+// and keys are multiplied by key_scale afterwards.  Queries are replaced in place.  With caches (key_caches / value_caches: device arrays [nseq] of pointers to
+// [positions][kv_heads * dim] and [positions][kv_heads * vdim], bf16 or f32) rotated keys and values go to row t of the sequence's caches; without (null) the
+// keys are replaced in place and values stay where they are.  kv_heads == 0: the row carries queries only (a layer that reads another layer's cache).
+struct RopeAppendParams {
+    float* qkv;
+    uint32_t ld, k_col, v_col;
+    uint32_t heads, kv_heads, dim, vdim, rope_dim;
+    const float *cosines, *sines;
+    float key_scale;
+    void* const* key_caches;
+    void* const* value_caches;
+    uint32_t cache_bf16;
+    const SeqSpan* spans;
+    const uint32_t* row_seq;
+    uint32_t rows;
+};
+uzu_status rope_append(hipStream_t s, const RopeAppendParams& p);
+
+// Attention over cached keys and values.  Row r (sequence z, position t), query head a, key / value head g = a / (heads / kv_heads):
+//   keys j = max(0, t - window + 1) .. t (window 0: from 0),  s_j = scale <q[r, a, :], K_z[j, g, :]>,  s_j <- cap tanh(s_j / cap) (cap != 0),
+//   p_j = exp(s_j - m) / (sum_j exp(s_j - m) + exp(sink_a - m))   (sinks f32 [heads] or null: no sink term),   out[r, a, :] = sum_j p_j V_z[j, g, :]
+// q f32 rows of pitch ldq (head a at column a * dim), out f32 [rows][heads * vdim]; caches as rope_append writes them.
+struct WindowAttentionParams {
+    const float* q;
+    uint32_t ldq;
+    float* out;
+    void* const* key_caches;
+    void* const* value_caches;
+    uint32_t cache_bf16;
+    const float* sinks;
+    const SeqSpan* spans;
+    const uint32_t* row_seq;
+    uint32_t rows, heads, kv_heads, dim, vdim, window;
+    float scale, soft_cap;
+    uint32_t form;  // 0: chosen by shape; 1: the simple form (a wave per row and head); 2: the matrix-core form
+    uint32_t nseq;  // entries of `spans`
+    uint32_t tiles; // sum over the sequences of ceil(count / 64): the matrix-core form's row tiles (the caller knows the counts)
+};
+bool window_attention_mfma_supported(const WindowAttentionParams& p);
+uzu_status window_attention(hipStream_t s, const WindowAttentionParams& p);
+
+// Retention.  Row r (sequence z, position t), head a, with q, k [heads][dim] and v [heads][vdim] taken from the f32 rows `qkv` (pitch ld; columns q_col, k_col,
+// v_col; q and k rotated and k scaled already):   S <- decay[a] S + k v^T,   out[r, a, :] = S^T q.
+// states: device array [nseq] of pointers to f32 [heads][dim][vdim], the sequences' states, read at the pass's first row (zero instead when the span starts at
+// position 0) and left behind its last.  Every sum runs in the same order whatever else the pass carries.  form 0: chosen by the sequence's row count; 1: token
+// by token; 2: in chunks of 64 rows (scores of the chunk's own rows + the carried state, a decayed state update per chunk).
+struct RetentionParams {
+    const float* qkv;
+    uint32_t ld, q_col, k_col, v_col;
+    float* out; // [rows][heads * vdim]
+    float* const* states;
+    const float* decay; // f32 [heads]
+    const SeqSpan* spans;
+    uint32_t nseq, rows, heads, dim, vdim;
+    uint32_t form;
+};
+bool retention_supported(uint32_t dim, uint32_t vdim);
+uzu_status retention(hipStream_t s, const RetentionParams& p);
+
+// Per head: x[r, a, :] <- x[r, a, :] / sqrt(mean(x[r, a, :]^2) + eps) * silu(gate[r, a * width ...])   (x f32 [rows][heads * width] in place; gate f32 rows of
+// pitch ldg; gate == null: the division alone)
+uzu_status head_rms_gate(hipStream_t s, float* x, const float* gate, uint32_t ldg, float eps, uint32_t rows, uint32_t heads, uint32_t width);
 
 } // namespace k
 } // namespace uzu

@@ -18,8 +18,8 @@ import numpy as np
 # enums (uzu_model_desc.h)
 QUANT_SCALE_BIAS, QUANT_SCALE_ZERO_POINT, QUANT_SCALE_SYMMETRIC, QUANT_NONE = 0, 1, 2, 3
 ACT_SILU, ACT_GELU_APPROX, ACT_GELU_EXACT, ACT_IDENTITY, ACT_SOFTPLUS, ACT_RELU_SQUARED = 0, 1, 2, 3, 4, 5
-MIXER_ATTENTION, MIXER_DELTA_NET, MIXER_LATENT_ATTENTION = 0, 1, 2
-NORM_STATISTICS, NORM_DYNAMIC_TANH = 0, 1
+MIXER_ATTENTION, MIXER_DELTA_NET, MIXER_LATENT_ATTENTION, MIXER_RETENTION = 0, 1, 2, 3
+NORM_STATISTICS, NORM_DYNAMIC_TANH, NORM_RMS_SCALAR = 0, 1, 2
 MOE_ROUTE_TOPK_LOGITS, MOE_ROUTE_SCORES = 0, 1
 ROPE_NONE, ROPE_UNSCALED, ROPE_LLAMA, ROPE_LINEAR, ROPE_YARN, ROPE_LONGROPE = 0, 1, 2, 3, 4, 5
 
@@ -63,6 +63,7 @@ class MoeDesc(C.Structure):
         ("gate_clip_min", C.c_float), ("gate_clip_max", C.c_float), ("up_clip_min", C.c_float), ("up_clip_max", C.c_float),
         ("router_weights", C.c_void_p), ("router_biases", C.c_void_p), ("w13", C.c_void_p), ("w2", C.c_void_p), ("up_biases", C.c_void_p), ("down_biases", C.c_void_p),
         ("routing", C.c_uint32), ("num_identity_experts", C.c_uint32), ("selection_bias", C.c_void_p),
+        ("up_offset", C.c_float), ("reserved", C.c_uint32),
     ]
 
 
@@ -95,7 +96,9 @@ class LayerDesc(C.Structure):
         ("latent_rank", C.c_uint32), ("value_head_dim", C.c_uint32),
         ("latent_down", LinearDesc), ("latent_norm", NormDesc), ("latent_up_keys", LinearDesc), ("latent_up_values", LinearDesc),
         ("token_shift", C.c_void_p), ("depth_weights", C.c_void_p),
-        ("num_depth_weights", C.c_uint32), ("mlp_plain", C.c_uint32), ("no_mlp", C.c_uint32), ("reserved4", C.c_uint32),
+        ("num_depth_weights", C.c_uint32), ("mlp_plain", C.c_uint32), ("no_mlp", C.c_uint32), ("parallel_block", C.c_uint32),
+        ("score_soft_cap", C.c_float), ("unit_sink", C.c_uint32), ("key_scale", C.c_float), ("head_norm_epsilon", C.c_float),
+        ("retention_decay", C.c_void_p), ("reserved4", C.c_uint32), ("reserved6", C.c_uint32),
     ]
 
 
@@ -176,7 +179,7 @@ class NormWeights:
     scale_offset: float = 0.0
     scales: Optional[np.ndarray] = None  # f32 [dim]
     biases: Optional[np.ndarray] = None
-    kind: int = NORM_STATISTICS          # NORM_DYNAMIC_TANH: tanh(alpha * x) * scales + biases (f32-stream designs)
+    kind: int = NORM_STATISTICS          # NORM_DYNAMIC_TANH: tanh(alpha * x) * scales + biases; NORM_RMS_SCALAR: alpha * x / sqrt(mean(x^2) + epsilon) (f32-stream designs)
     alpha: float = 0.0
 
     def desc(self) -> NormDesc:
@@ -232,11 +235,13 @@ class MoeWeights:
     routing: int = MOE_ROUTE_TOPK_LOGITS
     num_identity_experts: int = 0
     selection_bias: Optional[np.ndarray] = None  # f32 [E + identity]
+    up_offset: float = 0.0       # expert = down(act(gate) * (up + up_offset))
 
     def desc(self) -> MoeDesc:
         return MoeDesc(self.num_routed_experts, self.num_active_experts, self.expert_hidden_dim, int(self.router_renorm), self.gating_sel, self.silu_alpha,
                        self.gate_clip[0], self.gate_clip[1], self.up_clip[0], self.up_clip[1], _ptr(self.router_weights), _ptr(self.router_biases), _ptr(self.w13),
-                       _ptr(self.w2), _ptr(self.up_biases), _ptr(self.down_biases), int(self.routing), int(self.num_identity_experts), _ptr(self.selection_bias))
+                       _ptr(self.w2), _ptr(self.up_biases), _ptr(self.down_biases), int(self.routing), int(self.num_identity_experts), _ptr(self.selection_bias),
+                       float(self.up_offset), 0)
 
     def nbytes_active(self) -> int:
         """bytes one decoded token streams: the router + the k active experts' matrices and biases"""
@@ -304,6 +309,14 @@ class LayerWeights:
     depth_weights: Optional[np.ndarray] = None   # f32 [layer + 2]
     mlp_plain: bool = False
     no_mlp: bool = False
+    # f32-stream designs: parallel block (mixer and MLP read the same norm), attention with grouped heads / biases / rotation / score cap / window / sinks on a
+    # per-position cache of rotated keys and values (mixer_kind MIXER_ATTENTION), retention (MIXER_RETENTION: qkv_projection rows = q | k | v | gate)
+    parallel_block: bool = False
+    score_soft_cap: float = 0.0
+    unit_sink: bool = False
+    key_scale: float = 0.0
+    head_norm_epsilon: float = 0.0
+    retention_decay: Optional[np.ndarray] = None  # f32 [num_heads]
 
     def desc(self) -> LayerDesc:
         empty = LinearDesc()
@@ -330,7 +343,8 @@ class LayerWeights:
             (self.ple.norm if self.ple else ABSENT_NORM).desc(),
             self.moe.desc() if self.moe is not None else MoeDesc(),
             int(self.latent_rank), int(self.value_head_dim), ld(self.latent_down), self.latent_norm.desc(), ld(self.latent_up_keys), ld(self.latent_up_values),
-            _ptr(self.token_shift), _ptr(self.depth_weights), 0 if self.depth_weights is None else int(self.depth_weights.size), int(self.mlp_plain), int(self.no_mlp), 0,
+            _ptr(self.token_shift), _ptr(self.depth_weights), 0 if self.depth_weights is None else int(self.depth_weights.size), int(self.mlp_plain), int(self.no_mlp), int(self.parallel_block),
+            float(self.score_soft_cap), int(self.unit_sink), float(self.key_scale), float(self.head_norm_epsilon), _ptr(self.retention_decay), 0, 0,
         )
 
     def linears(self):

@@ -134,6 +134,16 @@ uzu_status uzu_hip_s32_latent_attention(uzu_hip_context* ctx, const float* qlat,
 uzu_status uzu_hip_s32_moe(uzu_hip_context* ctx, const float* x, const uint16_t* router, const float* selection_bias, const uint16_t* w13, const uint16_t* w2, const float* residual,
                            float* y, int32_t* ids_out, float* weights_out, uint32_t rows, uint32_t d, uint32_t ff, uint32_t routed, uint32_t identity, uint32_t top,
                            uint32_t bf16_products);
+/*   rotate: the first rope_dim coordinates of every query and key head of packed rows [queries | keys] turn by their position's angle (tables
+ *   [start + rows][rope_dim], both halves filled); keys are multiplied by key_scale afterwards.
+ *   window_attention: grouped heads over keys / values of positions 0 .. start + rows - 1, capped scores, causal window, sink logits; form 0 dispatch, 1 simple,
+ *   2 matrix cores.   retention: S <- decay S + k v^T, out = S^T q per head from state_inout (ignored at start 0); form 0 dispatch, 1 token by token, 2 chunks. */
+uzu_status uzu_hip_s32_rotate(uzu_hip_context* ctx, float* qk_inout, const float* cosines, const float* sines, uint32_t rows, uint32_t start, uint32_t heads, uint32_t kv_heads,
+                              uint32_t dim, uint32_t rope_dim, float key_scale);
+uzu_status uzu_hip_s32_window_attention(uzu_hip_context* ctx, const float* q, const float* keys, const float* values, const float* sinks, float* out, uint32_t rows, uint32_t start,
+                                        uint32_t heads, uint32_t kv_heads, uint32_t dim, uint32_t vdim, uint32_t window, float scale, float soft_cap, uint32_t cache_bf16, uint32_t form);
+uzu_status uzu_hip_s32_retention(uzu_hip_context* ctx, const float* q, const float* k, const float* v, const float* decay, float* state_inout, float* out, uint32_t rows,
+                                 uint32_t start, uint32_t heads, uint32_t dim, uint32_t vdim, uint32_t form);
 /* LanguageModelState reset: context length 0, DeltaNet conv / SSM state zeroed. */
 uzu_status uzu_hip_model_reset(uzu_hip_model* m);
 uint32_t uzu_hip_model_context_length(const uzu_hip_model* m);

@@ -1,6 +1,7 @@
 // capi_stream32.hip -- the kernels of the f32-stream designs behind plain C entries (include/uzu_hip_engine.h): host arrays in, host arrays out, ONE sequence.
 // They exist so that every mechanism can be held to an independent statement of its equations on its own (tests/test_gpu_lazolix_kernels.py) and so that two
 // forms of one kernel can be compared on the same inputs; the engine calls the kernels directly (engine_stream32.hip).
+#include <algorithm>
 #include <vector>
 
 #include "device_utils.h"
@@ -246,6 +247,110 @@ uzu_status uzu_hip_s32_moe(uzu_hip_context* ctx, const float* x, const uint16_t*
     UZU_HIP_TRY(hipMemcpy(y, dy, (size_t)rows * d * 4, hipMemcpyDeviceToHost));
     if (ids_out) UZU_HIP_TRY(hipMemcpy(ids_out, dids, (size_t)rows * top * 4, hipMemcpyDeviceToHost));
     if (weights_out) UZU_HIP_TRY(hipMemcpy(weights_out, dwt, (size_t)rows * top * 4, hipMemcpyDeviceToHost));
+    return UZU_OK;
+}
+
+// Rotation + key scaling in place on packed rows [rows][heads * dim (queries) + kv_heads * dim (keys)] at positions start ..; tables [start + rows][rope_dim]
+uzu_status uzu_hip_s32_rotate(uzu_hip_context* ctx, float* qk_inout, const float* cosines, const float* sines, uint32_t rows, uint32_t start, uint32_t heads, uint32_t kv_heads,
+                              uint32_t dim, uint32_t rope_dim, float key_scale) {
+    UZU_REQUIRE(ctx && qk_inout && cosines && sines, "s32_rotate: null argument");
+    (void)hipSetDevice(ctx->device);
+    Scratch S;
+    const uint32_t ld = (heads + kv_heads) * dim;
+    float *dx, *dc, *ds;
+    k::SeqSpan* spans;
+    uint32_t* row_seq;
+    UZU_PROPAGATE(S.up((const float*)qk_inout, (size_t)rows * ld, &dx));
+    UZU_PROPAGATE(S.up(cosines, (size_t)(start + rows) * rope_dim, &dc));
+    UZU_PROPAGATE(S.up(sines, (size_t)(start + rows) * rope_dim, &ds));
+    UZU_PROPAGATE(one_sequence(S, rows, start, &spans, &row_seq));
+    k::RopeAppendParams p{};
+    p.qkv = dx, p.ld = ld, p.k_col = heads * dim, p.v_col = ld, p.heads = heads, p.kv_heads = kv_heads, p.dim = dim, p.vdim = 0, p.rope_dim = rope_dim, p.cosines = dc, p.sines = ds;
+    p.key_scale = key_scale, p.spans = spans, p.row_seq = row_seq, p.rows = rows;
+    UZU_PROPAGATE(k::rope_append(ctx->stream, p));
+    UZU_PROPAGATE(finish(ctx));
+    UZU_HIP_TRY(hipMemcpy(qk_inout, dx, (size_t)rows * ld * 4, hipMemcpyDeviceToHost));
+    return UZU_OK;
+}
+
+// Attention of rows at positions start .. over keys [start + rows][kv_heads * dim] and values [start + rows][kv_heads * vdim] (f32 in; rounded to bf16 for a bf16
+// cache); q [rows][heads * dim] rotated already; sinks f32 [heads] or null.  form 0 dispatch, 1 simple, 2 matrix cores.
+uzu_status uzu_hip_s32_window_attention(uzu_hip_context* ctx, const float* q, const float* keys, const float* values, const float* sinks, float* out, uint32_t rows, uint32_t start,
+                                        uint32_t heads, uint32_t kv_heads, uint32_t dim, uint32_t vdim, uint32_t window, float scale, float soft_cap, uint32_t cache_bf16, uint32_t form) {
+    UZU_REQUIRE(ctx && q && keys && values && out && kv_heads, "s32_window_attention: null argument");
+    (void)hipSetDevice(ctx->device);
+    Scratch S;
+    float *dq, *dout, *dsink = nullptr;
+    void *dk = nullptr, *dv = nullptr;
+    void **dkp, **dvp;
+    k::SeqSpan* spans;
+    uint32_t* row_seq;
+    UZU_PROPAGATE(S.up(q, (size_t)rows * heads * dim, &dq));
+    UZU_PROPAGATE(S.up((const float*)nullptr, (size_t)rows * heads * vdim, &dout));
+    if (sinks) UZU_PROPAGATE(S.up(sinks, heads, &dsink));
+    auto cache = [&](const float* host, size_t total, void** dev) -> uzu_status {
+        if (cache_bf16) {
+            std::vector<uint16_t> bits(total);
+            for (size_t i = 0; i < total; ++i) bits[i] = f32_to_bf16(host[i]);
+            uint16_t* d16;
+            UZU_PROPAGATE(S.up(bits.data(), total, &d16));
+            *dev = d16;
+        } else {
+            float* d32;
+            UZU_PROPAGATE(S.up(host, total, &d32));
+            *dev = d32;
+        }
+        return UZU_OK;
+    };
+    UZU_PROPAGATE(cache(keys, (size_t)(start + rows) * kv_heads * dim, &dk));
+    UZU_PROPAGATE(cache(values, (size_t)(start + rows) * kv_heads * vdim, &dv));
+    UZU_PROPAGATE(S.up((void* const*)&dk, 1, &dkp));
+    UZU_PROPAGATE(S.up((void* const*)&dv, 1, &dvp));
+    UZU_PROPAGATE(one_sequence(S, rows, start, &spans, &row_seq));
+    k::WindowAttentionParams p{};
+    p.q = dq, p.ldq = heads * dim, p.out = dout, p.key_caches = dkp, p.value_caches = dvp, p.cache_bf16 = cache_bf16, p.sinks = dsink, p.spans = spans, p.row_seq = row_seq;
+    p.rows = rows, p.heads = heads, p.kv_heads = kv_heads, p.dim = dim, p.vdim = vdim, p.window = window, p.scale = scale, p.soft_cap = soft_cap, p.form = form, p.nseq = 1;
+    p.tiles = heads % kv_heads == 0 ? (rows * (heads / kv_heads) + 127) / 128 : 0;
+    UZU_PROPAGATE(k::window_attention(ctx->stream, p));
+    UZU_PROPAGATE(finish(ctx));
+    UZU_HIP_TRY(hipMemcpy(out, dout, (size_t)rows * heads * vdim * 4, hipMemcpyDeviceToHost));
+    return UZU_OK;
+}
+
+// Retention of rows at positions start ..: q, k [rows][heads * dim] (rotated, scaled), v [rows][heads * vdim], decay [heads]; state_inout [heads][dim][vdim] is the
+// state in front of the rows (ignored when start == 0) and behind them.  form 0 dispatch, 1 token by token, 2 in chunks.
+uzu_status uzu_hip_s32_retention(uzu_hip_context* ctx, const float* q, const float* kk, const float* v, const float* decay, float* state_inout, float* out, uint32_t rows, uint32_t start,
+                                 uint32_t heads, uint32_t dim, uint32_t vdim, uint32_t form) {
+    UZU_REQUIRE(ctx && q && kk && v && decay && state_inout && out, "s32_retention: null argument");
+    (void)hipSetDevice(ctx->device);
+    Scratch S;
+    const uint32_t ld = heads * (2 * dim + vdim);
+    std::vector<float> packed((size_t)rows * ld);
+    for (uint32_t r = 0; r < rows; ++r) {
+        std::copy(q + (size_t)r * heads * dim, q + (size_t)(r + 1) * heads * dim, packed.begin() + (size_t)r * ld);
+        std::copy(kk + (size_t)r * heads * dim, kk + (size_t)(r + 1) * heads * dim, packed.begin() + (size_t)r * ld + heads * dim);
+        std::copy(v + (size_t)r * heads * vdim, v + (size_t)(r + 1) * heads * vdim, packed.begin() + (size_t)r * ld + 2 * heads * dim);
+    }
+    float *dx, *dd, *dst, *dout, *dws = nullptr;
+    float** dsp;
+    k::SeqSpan* spans;
+    uint32_t* row_seq;
+    UZU_PROPAGATE(S.up(packed.data(), packed.size(), &dx));
+    UZU_PROPAGATE(S.up(decay, heads, &dd));
+    UZU_PROPAGATE(S.up((const float*)state_inout, (size_t)heads * dim * vdim, &dst));
+    UZU_PROPAGATE(S.up((const float*)nullptr, (size_t)rows * heads * vdim, &dout));
+    UZU_PROPAGATE(S.up((float* const*)&dst, 1, &dsp));
+    UZU_PROPAGATE(one_sequence(S, rows, start, &spans, &row_seq));
+    k::RetentionParams p{};
+    p.qkv = dx, p.ld = ld, p.q_col = 0, p.k_col = heads * dim, p.v_col = 2 * heads * dim, p.out = dout, p.states = dsp, p.decay = dd, p.spans = spans, p.nseq = 1, p.rows = rows;
+    p.heads = heads, p.dim = dim, p.vdim = vdim, p.form = form, p.chunks = (rows + 63) / 64;
+    p.chunk_ws_bytes = k::retention_chunk_ws_bytes(p.chunks, heads, dim, vdim);
+    UZU_PROPAGATE(S.up((const float*)nullptr, p.chunk_ws_bytes / 4, &dws));
+    p.chunk_ws = dws;
+    UZU_PROPAGATE(k::retention(ctx->stream, p));
+    UZU_PROPAGATE(finish(ctx));
+    UZU_HIP_TRY(hipMemcpy(out, dout, (size_t)rows * heads * vdim * 4, hipMemcpyDeviceToHost));
+    UZU_HIP_TRY(hipMemcpy(state_inout, dst, (size_t)heads * dim * vdim * 4, hipMemcpyDeviceToHost));
     return UZU_OK;
 }
 

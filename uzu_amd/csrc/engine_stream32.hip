@@ -54,6 +54,8 @@ struct Stream32 {
     };
     std::vector<Layer> layers;
     float alpha_out = 0.f;
+    float* ret_ws = nullptr; // retention in chunks: one state block per (chunk of the pass, head)
+    size_t ret_ws_bytes = 0;
     float* att_ws = nullptr; // partial sums of the key-split attention of decode-sized passes
     size_t att_ws_bytes = 0;
     float* taps = nullptr; // UZU_MODEL_DEBUG_TAPS: f32 [layers][max_rows][d], what each layer handed on in the last pass
@@ -213,7 +215,7 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
             ap.q = S.q, ap.ldq = ldq, ap.out = S.attn, ap.key_caches = caches, ap.value_caches = vcaches, ap.cache_bf16 = bf, ap.sinks = X.sinks, ap.spans = S.d_spans;
             ap.row_seq = S.d_row_seq, ap.rows = rows, ap.heads = H, ap.kv_heads = G, ap.dim = hd, ap.vdim = vd, ap.window = h.sliding_window_size;
             ap.scale = h.attention_scale != 0.0f ? h.attention_scale : 1.0f / sqrtf((float)hd), ap.soft_cap = h.score_soft_cap, ap.nseq = nseq;
-            for (uint32_t i = 0; i < nseq; ++i) ap.tiles += (counts[i] + 63) / 64;
+            for (uint32_t i = 0; i < nseq; ++i) ap.tiles += (counts[i] * (H / G) + 127) / 128;
             RUN("window_attention", (size_t)rows * H * (hd + vd) * 4, k::window_attention(s, ap));
         } else if (h.mixer_kind == UZU_MIXER_RETENTION) {
             const uint32_t ldq = L.qkv.n; // queries | keys | values | gate
@@ -225,6 +227,8 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
             k::RetentionParams tp{};
             tp.qkv = S.q, tp.ld = ldq, tp.q_col = 0, tp.k_col = H * hd, tp.v_col = 2 * H * hd, tp.out = S.attn, tp.states = (float* const*)caches, tp.decay = X.decay;
             tp.spans = S.d_spans, tp.nseq = nseq, tp.rows = rows, tp.heads = H, tp.dim = hd, tp.vdim = vd;
+            for (uint32_t i = 0; i < nseq; ++i) tp.chunks += (counts[i] + 63) / 64;
+            tp.chunk_ws = S.ret_ws, tp.chunk_ws_bytes = S.ret_ws_bytes;
             RUN("retention", (size_t)rows * ldq * 4 + (size_t)nseq * H * hd * vd * 8, k::retention(s, tp));
             RUN("head_rms_gate", (size_t)rows * H * vd * 12, k::head_rms_gate(s, S.attn, S.q + 2 * H * hd + H * vd, ldq, h.head_norm_epsilon, rows, H, vd));
         } else {
@@ -604,6 +608,12 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
         S.att_ws_bytes = k::latent_attention_split_ws_bytes(std::min<uint32_t>(4 * S.max_seqs, 4096 / hmax ? 4096 / hmax : 1), hmax, 256, 32);
         TRY(need_f32(m, S.att_ws_bytes / 4, &S.att_ws));
     }
+    for (uint32_t l = 0; l < nl; ++l) {
+        const uzu_layer_desc& h = desc->layers[l];
+        if (h.mixer_kind == UZU_MIXER_RETENTION)
+            S.ret_ws_bytes = std::max(S.ret_ws_bytes, k::retention_chunk_ws_bytes(S.max_rows / 64 + S.max_seqs, h.num_heads, h.head_dim, h.value_head_dim));
+    }
+    if (S.ret_ws_bytes) TRY(need_f32(m, S.ret_ws_bytes / 4, &S.ret_ws));
     TRY(dev_alloc(m, k::argmax_scratch_bytes(1), &m->argmax_scratch));
     TRY(dev_alloc(m, k::unified_sampling_scratch_bytes(1), &m->sampling_scratch));
     TRY(dev_alloc(m, 8, &p, true)); m->d_seed = (uint64_t*)p;

@@ -188,7 +188,7 @@ struct WindowAttentionParams {
     float scale, soft_cap;
     uint32_t form;  // 0: chosen by shape; 1: the simple form (a wave per row and head); 2: the matrix-core form
     uint32_t nseq;  // entries of `spans`
-    uint32_t tiles; // sum over the sequences of ceil(count / 64): the matrix-core form's row tiles (the caller knows the counts)
+    uint32_t tiles; // sum over the sequences of ceil(count * (heads / kv_heads) / 128): the matrix-core form's item tiles (the caller knows the counts)
 };
 bool window_attention_mfma_supported(const WindowAttentionParams& p);
 uzu_status window_attention(hipStream_t s, const WindowAttentionParams& p);
@@ -207,7 +207,13 @@ struct RetentionParams {
     const SeqSpan* spans;
     uint32_t nseq, rows, heads, dim, vdim;
     uint32_t form;
+    // the chunked form: chunks = sum over the sequences of ceil(count / 64) (the caller knows the counts) and a workspace of
+    // retention_chunk_ws_bytes(chunks, heads, dim, vdim) bytes; without one, form 0 goes token by token
+    uint32_t chunks;
+    float* chunk_ws;
+    size_t chunk_ws_bytes;
 };
+size_t retention_chunk_ws_bytes(uint32_t chunks, uint32_t heads, uint32_t dim, uint32_t vdim);
 bool retention_supported(uint32_t dim, uint32_t vdim);
 uzu_status retention(hipStream_t s, const RetentionParams& p);
 

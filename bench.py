@@ -12,8 +12,8 @@ Prints ONE JSON line on rank 0 (contract in the task statement) with two extra o
   roofline     -- the dominant kernel (the int4 GEMV family) : algorithmic bytes / HIP-event time, vs 8 TB/s HBM
   cpu_baseline -- the CPU oracle (port of the reference's single-threaded CPU backend) timed on this host
 
-Side runs (their own JSON line, never the headline): --config c3|c4|c5, --exact, and --design lazolix (prefill / chained decode / batched decode of the
-f32-stream design at real layer sizes beside the closest bf16-stream model of the engine).
+Side runs (their own JSON line, never the headline): --config c3|c4|c5, --exact, and --design lazolix | relulix (prefill / chained decode / batched
+decode of an f32-stream design at real layer sizes beside the engine's closest existing model at equal sizes).
 """
 import argparse
 import dataclasses
@@ -59,9 +59,10 @@ def parse_args():
                     help="BASELINE.json configs[1..4]: c2 (default, the headline) Qwen3.5-0.8B int4 ctx-2048 decode; c3 Llama-3-8B int4, 4k prefill x 8 "
                          "sequences in batched passes (prefill tokens/s, MFMA roofline); c4 Llama-3-8B int8 decode (TP = --gpus); c5 Qwen3-14B-class int4 at "
                          "ctx 8192, one sequence decoding while another is prefilled (TP = --gpus)")
-    ap.add_argument("--design", choices=["", "lazolix"], default="", help="side runs of a design outside BASELINE.json (never the headline): `lazolix` times prefill, "
+    ap.add_argument("--design", choices=["", "lazolix", "relulix"], default="", help="side runs of a design outside BASELINE.json (never the headline): `lazolix` times prefill, "
                     "chained decode and batched decode of the f32-stream design at layer sizes of real models (random weights), beside the closest "
-                    "bf16-stream model of the engine at equal sizes (windowed attention with sinks + int4 dense / bf16 expert MLPs)")
+                    "bf16-stream model of the engine at equal sizes (windowed attention with sinks + int4 dense / bf16 expert MLPs); `relulix` does the same for the "
+                    "design of parallel blocks with rotated attention, retention layers and clamped experts, beside Lazolix with experts at equal sizes")
     ap.add_argument("--design-sizes", default="w1024,w2048", help="--design: comma-separated size presets")
     ap.add_argument("--sequences", type=int, default=8, help="c3: sequences per batched prefill pass")
     ap.add_argument("--prompt", type=int, default=4096, help="c3: prompt tokens per sequence")
@@ -472,61 +473,73 @@ LAZOLIX_SIZES = {  # layer sizes of real models: width, heads x (dim, vdim), lat
 }
 
 
+def _time_f32_stream(ctx, bundle, prompt, steps, warm, nbatch):
+    """prefill / chained decode / batched decode of one f32-stream model (HipModel.prefill, decode, step_batch)"""
+    from uzu_amd.engine import MODEL_BATCH, HipModel
+    prompt_len = len(prompt)
+    m = HipModel(ctx, bundle, MODEL_BATCH(nbatch))
+
+    def prefill():
+        m.reset()
+        m.prefill(prompt)
+    t_prefill = _timed(ctx, prefill)
+    m.decode(warm)
+    t0 = time.perf_counter()
+    m.decode(steps)
+    ctx.synchronize()
+    t_decode = time.perf_counter() - t0
+    states = [m.new_state() for _ in range(nbatch)]
+    m.step_batch(states, [list(prompt)] * nbatch, None)
+    step = lambda: m.step_batch(states, [[7]] * nbatch, None, sample=True)
+    t_batch = _timed(ctx, step, reps=8)
+    rec = {"prefill_tokens_per_s": round(prompt_len / t_prefill, 1), "prefill_tflops": round(bundle.prefill_flops(prompt_len) / t_prefill / 1e12, 2),
+           "decode_tokens_per_s": round(steps / t_decode, 1), "decode_us_per_token": round(t_decode / steps * 1e6, 1),
+           "decode_launches": m.decode_launch_count, "decode_gbps": round(bundle.decode_bytes_per_token(prompt_len) * steps / t_decode / 1e9, 1),
+           "batched_decode_tokens_per_s": round(nbatch / t_batch, 1), "weight_bytes": m.weight_bytes}
+    for st in states:
+        st.close()
+    m.close()
+    return rec
+
+
+def _timed(ctx, fn, reps=3):
+    fn()
+    ctx.synchronize()
+    best = 1e30
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        fn()
+        ctx.synchronize()
+        best = min(best, time.perf_counter() - t0)
+    return best
+
+
+def _lazolix_bundle(z, kind, context):
+    import tempfile
+    from uzu_amd import lazolix, loader
+    mlp = lazolix.dense_mlp(z["ff"]) if kind == "dense" else lazolix.moe_mlp(z["experts"], z["top"], z["eff"], z["identity"])
+    layers = [lazolix.layer_config(z["heads"], z["dim"], z["vdim"], z["rank"], z["window"], kv_from=(l - 1 if l % 2 else None), mlp=mlp) for l in range(z["layers"])]
+    cfg = {"vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-6}, "layers": layers}
+    with tempfile.TemporaryDirectory() as tmp:
+        lazolix.save(tmp, cfg, lazolix.random_tensors(cfg, seed=1))
+        return loader.load_model_dir(tmp, max_context_length=context)
+
+
 def bench_lazolix(args):
     """Prefill / decode throughput of Lazolix models (dense and expert MLPs) and of the closest bf16-stream model at the same sizes.  One JSON line."""
-    import tempfile
-    from uzu_amd import desc as D, lazolix, loader, synthetic as S
+    from uzu_amd import desc as D, synthetic as S
     from uzu_amd.backend import Context
-    from uzu_amd.engine import MODEL_BATCH, MODEL_DEFAULT, HipModel
+    from uzu_amd.engine import MODEL_DEFAULT, HipModel
     ctx = Context.new(0)
     prompt_len, steps, warm, nbatch = 2048, max(8, min(args.steps, 128)), max(2, min(args.warmup, 8)), 8
     out = {"metric": "lazolix_side_run", "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16 products, f32 stream", "data": "synthetic (random weights, synthetic token ids)",
            "prompt_tokens": prompt_len, "decode_steps": steps, "batched_decode_sequences": nbatch, "sizes": {}}
-
-    def timed(fn, reps=3):
-        fn()
-        ctx.synchronize()
-        best = 1e30
-        for _ in range(reps):
-            t0 = time.perf_counter()
-            fn()
-            ctx.synchronize()
-            best = min(best, time.perf_counter() - t0)
-        return best
-
     for size in [s for s in args.design_sizes.split(",") if s]:
         z = LAZOLIX_SIZES[size]
         rec = {}
         prompt = S.synthetic_prompt(prompt_len, z["vocab"]).astype(np.uint32)
         for kind in ("dense", "moe"):
-            mlp = lazolix.dense_mlp(z["ff"]) if kind == "dense" else lazolix.moe_mlp(z["experts"], z["top"], z["eff"], z["identity"])
-            layers = [lazolix.layer_config(z["heads"], z["dim"], z["vdim"], z["rank"], z["window"], kv_from=(l - 1 if l % 2 else None), mlp=mlp) for l in range(z["layers"])]
-            cfg = {"vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-6}, "layers": layers}
-            with tempfile.TemporaryDirectory() as tmp:
-                lazolix.save(tmp, cfg, lazolix.random_tensors(cfg, seed=1))
-                bundle = loader.load_model_dir(tmp, max_context_length=prompt_len + steps + warm + 64)
-            m = HipModel(ctx, bundle, MODEL_BATCH(nbatch))
-
-            def prefill():
-                m.reset()
-                m.prefill(prompt)
-            t_prefill = timed(prefill)
-            m.decode(warm)
-            t0 = time.perf_counter()
-            m.decode(steps)
-            ctx.synchronize()
-            t_decode = time.perf_counter() - t0
-            states = [m.new_state() for _ in range(nbatch)]
-            m.step_batch(states, [list(prompt)] * nbatch, None)
-            step = lambda: m.step_batch(states, [[7]] * nbatch, None, sample=True)
-            t_batch = timed(step, reps=8)
-            rec["lazolix_" + kind] = {"prefill_tokens_per_s": round(prompt_len / t_prefill, 1), "prefill_tflops": round(bundle.prefill_flops(prompt_len) / t_prefill / 1e12, 2),
-                                      "decode_tokens_per_s": round(steps / t_decode, 1), "decode_us_per_token": round(t_decode / steps * 1e6, 1),
-                                      "decode_launches": m.decode_launch_count, "decode_gbps": round(bundle.decode_bytes_per_token(prompt_len) * steps / t_decode / 1e9, 1),
-                                      "batched_decode_tokens_per_s": round(nbatch / t_batch, 1), "weight_bytes": m.weight_bytes}
-            for st in states:
-                st.close()
-            m.close()
+            rec["lazolix_" + kind] = _time_f32_stream(ctx, _lazolix_bundle(z, kind, prompt_len + steps + warm + 64), prompt, steps, warm, nbatch)
             # the closest bf16-stream model: windowed attention with sinks, same width / heads / head width / layers / vocabulary; int4 g128 dense MLP of the same
             # hidden width, or bf16 experts of the same count and width
             ccfg = S.ModelConfig(name=f"closest-{size}-{kind}", vocab_size=z["vocab"], model_dim=z["width"], hidden_dim=z["ff"], layer_kinds=[D.MIXER_ATTENTION] * z["layers"],
@@ -540,7 +553,7 @@ def bench_lazolix(args):
             def cprefill():
                 cm.reset()
                 cm.prefill(prompt)
-            ct_prefill = timed(cprefill)
+            ct_prefill = _timed(ctx, cprefill)
             cm.decode(warm)
             t0 = time.perf_counter()
             cm.decode(steps)
@@ -556,10 +569,44 @@ def bench_lazolix(args):
     print(json.dumps(out), flush=True)
 
 
+def bench_relulix(args):
+    """Prefill / decode throughput of Relulix models (parallel blocks: three attention layers, one of them on a shared cache, and a retention layer; routed
+    experts) beside the closest existing model at equal size: Lazolix with experts (the other f32-stream design: windowed attention with a sink, routed
+    experts; same width / heads / head widths / window / experts / layers / vocabulary).  One JSON line."""
+    import tempfile
+    from uzu_amd import loader, relulix, synthetic as S
+    from uzu_amd.backend import Context
+    ctx = Context.new(0)
+    prompt_len, steps, warm, nbatch = 2048, max(8, min(args.steps, 128)), max(2, min(args.warmup, 8)), 8
+    out = {"metric": "relulix_side_run", "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16 products, f32 stream", "data": "synthetic (random weights, synthetic token ids)",
+           "prompt_tokens": prompt_len, "decode_steps": steps, "batched_decode_sequences": nbatch, "sizes": {}}
+    for size in [s for s in args.design_sizes.split(",") if s]:
+        z = LAZOLIX_SIZES[size]
+        prompt = S.synthetic_prompt(prompt_len, z["vocab"]).astype(np.uint32)
+        context = prompt_len + steps + warm + 64
+        H, G, dim, vd = z["heads"], max(1, z["heads"] // 4), z["dim"], z["vdim"]
+        yarn = {"factor": 8.0, "original": 4096, "fast": 16.0, "slow": 2.0}
+        mlp = relulix.moe_mlp(z["experts"], z["top"], z["eff"], limit=7.0)
+        att = lambda kv_from=None: relulix.attention_layer(H, G, dim, vd, relulix.rotation(dim // 2, 10000.0, yarn), window=z["window"], softcap=30.0, kv_from=kv_from, mlp=mlp)
+        ret = relulix.retention_layer(H, dim, vd, relulix.rotation(dim, 1e6), [1.0 - 2.0 ** -(5 + (a % 6)) for a in range(H)], mlp=mlp)
+        layers = ([att(), att(0), att(), ret] * ((z["layers"] + 3) // 4))[:z["layers"]]
+        cfg = relulix.config(z["vocab"], z["width"], layers)
+        with tempfile.TemporaryDirectory() as tmp:
+            relulix.save(tmp, cfg, relulix.random_tensors(cfg, seed=1))
+            bundle = loader.load_model_dir(tmp, max_context_length=context)
+        rec = {"relulix_moe": _time_f32_stream(ctx, bundle, prompt, steps, warm, nbatch),
+               "closest_moe": _time_f32_stream(ctx, _lazolix_bundle(z, "moe", context), prompt, steps, warm, nbatch)}
+        out["sizes"][size] = {"shape": dict(z, kv_heads=G, pattern="attention, attention on layer 0's cache, attention, retention"), **rec}
+    ctx.close()
+    print(json.dumps(out), flush=True)
+
+
 def main():
     args = parse_args()
     if args.design == "lazolix":
         return bench_lazolix(args)
+    if args.design == "relulix":
+        return bench_relulix(args)
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ and not args.force_dist:
         spawn_ranks(args.gpus)
     if args.config == "c3":

@@ -553,7 +553,9 @@ class ModelBundle:
         for l in self.layers:
             if l.mixer_kind == MIXER_ATTENTION:
                 rows = min(context, l.sliding_window_size) if l.sliding_window_size else context
-                total += 2 * rows * l.num_groups * l.head_dim * 2             # K and V rows, bf16 (a sharing layer reads its source's)
+                total += rows * l.num_groups * (l.head_dim + (l.value_head_dim or l.head_dim)) * 2  # K and V rows, bf16 (a sharing layer reads its source's)
+            elif l.mixer_kind == MIXER_RETENTION:
+                total += 2 * l.num_heads * l.head_dim * l.value_head_dim * 4  # f32 state read + write
             elif l.mixer_kind == MIXER_LATENT_ATTENTION:
                 rows = min(context, l.sliding_window_size) if l.sliding_window_size else context
                 total += rows * l.latent_rank * 2                             # one latent row per visible token, bf16, shared by all heads
@@ -579,8 +581,14 @@ class ModelBundle:
         flops += 2.0 * readout.n * readout.k
         pairs = tokens * context_before + tokens * (tokens + 1) / 2.0
         for l in self.layers:
-            if l.mixer_kind == MIXER_ATTENTION:
+            if l.mixer_kind == MIXER_ATTENTION and l.value_head_dim:  # an f32-stream design's attention: its own value width, the window counted
+                w = l.sliding_window_size
+                vis = pairs if not w else min(pairs, tokens * float(w))
+                flops += 2.0 * vis * l.num_heads * (l.head_dim + l.value_head_dim)
+            elif l.mixer_kind == MIXER_ATTENTION:
                 flops += 4.0 * pairs * l.num_heads * l.head_dim
+            elif l.mixer_kind == MIXER_RETENTION:  # per token and head: the outer-product update and the read-out of the state
+                flops += 4.0 * tokens * l.num_heads * l.head_dim * l.value_head_dim
             elif l.mixer_kind == MIXER_LATENT_ATTENTION:  # scores and weighted sum in latent space, over the window
                 w = l.sliding_window_size
                 vis = pairs if not w else min(pairs, tokens * float(w))

@@ -137,7 +137,7 @@ uzu_status uzu_hip_s32_moe(uzu_hip_context* ctx, const float* x, const uint16_t*
 /*   rotate: the first rope_dim coordinates of every query and key head of packed rows [queries | keys] turn by their position's angle (tables
  *   [start + rows][rope_dim], both halves filled); keys are multiplied by key_scale afterwards.
  *   window_attention: grouped heads over keys / values of positions 0 .. start + rows - 1, capped scores, causal window, sink logits; form 0 dispatch, 1 simple,
- *   2 matrix cores.   retention: S <- decay S + k v^T, out = S^T q per head from state_inout (ignored at start 0); form 0 dispatch, 1 token by token, 2 chunks. */
+ *   2 matrix cores, 3 matrix cores with the keys split over workgroups.   retention: S <- decay S + k v^T, out = S^T q per head from state_inout (ignored at start 0); form 0 dispatch, 1 token by token, 2 chunks. */
 uzu_status uzu_hip_s32_rotate(uzu_hip_context* ctx, float* qk_inout, const float* cosines, const float* sines, uint32_t rows, uint32_t start, uint32_t heads, uint32_t kv_heads,
                               uint32_t dim, uint32_t rope_dim, float key_scale);
 uzu_status uzu_hip_s32_window_attention(uzu_hip_context* ctx, const float* q, const float* keys, const float* values, const float* sinks, float* out, uint32_t rows, uint32_t start,

@@ -109,6 +109,18 @@ def test_attention_matrix_core_form_equals_the_simple_form(hip_ctx, H, G, dim, v
     assert np.abs(a - want).max() < 6e-5 * np.abs(want).max()  # the query as hi + lo bf16: 16 significant bits
 
 
+@pytest.mark.parametrize("H,G,dim,vd,window,cap,T,start", [c for c in CASES if c[2] % 8 == 0 and c[3] % 8 == 0])
+def test_attention_split_keys_form_on_few_rows(hip_ctx, H, G, dim, vd, window, cap, T, start):
+    """a decode-sized pass: the last one to three rows of the sequence, their key blocks spread over five workgroups and merged"""
+    rng = np.random.default_rng(H * 100 + T + 2)
+    q, K, V = qkv(rng, T, H, G, dim, vd)
+    mx = {"heads": H, "kv_heads": G, "scale": 1.7 / np.sqrt(dim), "mask": {"size": window}, "softcap": cap}
+    for rows in (1, 3):
+        want = O.attention_core(f32(q)[T - rows:], O.to_bf16(K), O.to_bf16(V), mx, T - rows)
+        got = attention(hip_ctx, q[T - rows:], K, V, mx, T - rows, bf16=1, form=3)
+        assert np.isfinite(got).all() and np.abs(got - want).max() < 6e-5 * np.abs(want).max()
+
+
 @pytest.mark.parametrize("bf16,form", [(0, 1), (1, 1), (1, 2)])
 @pytest.mark.parametrize("window", [1, 2, 31, 32, 33, 64, 65, 130])
 def test_one_key_stands_out_just_inside_and_just_outside_the_window(hip_ctx, bf16, form, window):
@@ -130,7 +142,7 @@ def test_one_key_stands_out_just_inside_and_just_outside_the_window(hip_ctx, bf1
             q2[t, :, 3] = 8.0       # score 64 against O(1) elsewhere
             V2[j, 0] = 100.0 + np.arange(vd)
             for start in (0, t):    # the row inside a prompt from position 0, and decoded alone
-                got = attention(hip_ctx, q2[start:t + 1], K2[:t + 1], V2[:t + 1], mx, start, bf16=bf16, form=form if (start == 0 and t + 1 >= 16) else 1)[-1]
+                got = attention(hip_ctx, q2[start:t + 1], K2[:t + 1], V2[:t + 1], mx, start, bf16=bf16, form=form if (start == 0 and t + 1 >= 16) else (3 if form == 2 else 1))[-1]
                 if inside:
                     assert np.abs(got - V2[j, 0]).max() < 1e-2, (t, start)
                 else:

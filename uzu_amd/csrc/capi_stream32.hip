@@ -274,7 +274,7 @@ uzu_status uzu_hip_s32_rotate(uzu_hip_context* ctx, float* qk_inout, const float
 }
 
 // Attention of rows at positions start .. over keys [start + rows][kv_heads * dim] and values [start + rows][kv_heads * vdim] (f32 in; rounded to bf16 for a bf16
-// cache); q [rows][heads * dim] rotated already; sinks f32 [heads] or null.  form 0 dispatch, 1 simple, 2 matrix cores.
+// cache); q [rows][heads * dim] rotated already; sinks f32 [heads] or null.  form 0 dispatch, 1 simple, 2 matrix cores, 3 matrix cores with split keys.
 uzu_status uzu_hip_s32_window_attention(uzu_hip_context* ctx, const float* q, const float* keys, const float* values, const float* sinks, float* out, uint32_t rows, uint32_t start,
                                         uint32_t heads, uint32_t kv_heads, uint32_t dim, uint32_t vdim, uint32_t window, float scale, float soft_cap, uint32_t cache_bf16, uint32_t form) {
     UZU_REQUIRE(ctx && q && keys && values && out && kv_heads, "s32_window_attention: null argument");
@@ -311,6 +311,13 @@ uzu_status uzu_hip_s32_window_attention(uzu_hip_context* ctx, const float* q, co
     p.q = dq, p.ldq = heads * dim, p.out = dout, p.key_caches = dkp, p.value_caches = dvp, p.cache_bf16 = cache_bf16, p.sinks = dsink, p.spans = spans, p.row_seq = row_seq;
     p.rows = rows, p.heads = heads, p.kv_heads = kv_heads, p.dim = dim, p.vdim = vdim, p.window = window, p.scale = scale, p.soft_cap = soft_cap, p.form = form, p.nseq = 1;
     p.tiles = heads % kv_heads == 0 ? (rows * (heads / kv_heads) + 127) / 128 : 0;
+    if (form == 3) { // the matrix-core form with its key blocks split over workgroups + the merge launch
+        float* ws = nullptr;
+        p.form = 2, p.splits = 5;
+        p.split_ws_bytes = k::window_attention_split_ws_bytes(rows, heads, p.splits);
+        UZU_PROPAGATE(S.up((const float*)nullptr, p.split_ws_bytes / 4, &ws));
+        p.split_ws = ws;
+    }
     UZU_PROPAGATE(k::window_attention(ctx->stream, p));
     UZU_PROPAGATE(finish(ctx));
     UZU_HIP_TRY(hipMemcpy(out, dout, (size_t)rows * heads * vdim * 4, hipMemcpyDeviceToHost));

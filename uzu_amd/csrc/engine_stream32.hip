@@ -216,6 +216,9 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
             ap.row_seq = S.d_row_seq, ap.rows = rows, ap.heads = H, ap.kv_heads = G, ap.dim = hd, ap.vdim = vd, ap.window = h.sliding_window_size;
             ap.scale = h.attention_scale != 0.0f ? h.attention_scale : 1.0f / sqrtf((float)hd), ap.soft_cap = h.score_soft_cap, ap.nseq = nseq;
             for (uint32_t i = 0; i < nseq; ++i) ap.tiles += (counts[i] * (H / G) + 127) / 128;
+            // decode-sized passes: spread a tile's key blocks over workgroups (a constant of the layer, so that a captured step stays valid as the context grows)
+            const uint32_t keys = h.sliding_window_size ? h.sliding_window_size : m->d.max_context_length;
+            if (rows <= 4 * S.max_seqs && rows * H <= 4096) ap.splits = std::min<uint32_t>(16, (keys + 31) / 32), ap.split_ws = S.att_ws, ap.split_ws_bytes = S.att_ws_bytes;
             RUN("window_attention", (size_t)rows * H * (hd + vd) * 4, k::window_attention(s, ap));
         } else if (h.mixer_kind == UZU_MIXER_RETENTION) {
             const uint32_t ldq = L.qkv.n; // queries | keys | values | gate
@@ -605,7 +608,8 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
     {
         uint32_t hmax = 0;
         for (uint32_t l = 0; l < nl; ++l) hmax = std::max(hmax, desc->layers[l].num_heads);
-        S.att_ws_bytes = k::latent_attention_split_ws_bytes(std::min<uint32_t>(4 * S.max_seqs, 4096 / hmax ? 4096 / hmax : 1), hmax, 256, 32);
+        const uint32_t few = std::min<uint32_t>(4 * S.max_seqs, 4096 / hmax ? 4096 / hmax : 1);
+        S.att_ws_bytes = std::max(k::latent_attention_split_ws_bytes(few, hmax, 256, 32), k::window_attention_split_ws_bytes(few, hmax, 16));
         TRY(need_f32(m, S.att_ws_bytes / 4, &S.att_ws));
     }
     for (uint32_t l = 0; l < nl; ++l) {

@@ -4,6 +4,8 @@
 // Token by token (this file's first kernel): a workgroup per (sequence, head) keeps the state in registers -- thread (j, part) owns S[i][j] for the rows
 // i = part, part + parts, ... -- so the update and the thread's share of S^T q touch no memory; the shares of a column meet in LDS and are added in a fixed
 // order.  The same kernel runs prompts and decode steps, so a prompt's state does not depend on how it was cut.
+#include <algorithm>
+
 #include "device_utils.h"
 #include "kernels_stream32.h"
 
@@ -136,7 +138,7 @@ __global__ void __launch_bounds__(256) retention_chunk_scan_kernel(RetentionPara
     for (uint32_t t = 0; t < kChunk; ++t) pw_full *= decay;
     float pw_last = 1.0f;
     for (uint32_t t = 0; t < sp.count - (chunks - 1) * kChunk; ++t) pw_last *= decay;
-    for (uint32_t e = threadIdx.x; e < elems; e += 256) {
+    for (uint32_t e = blockIdx.z * 256 + threadIdx.x; e < elems; e += 256 * gridDim.z) { // the elements are independent of each other: one per thread
         float S = sp.start ? state[e] : 0.0f;
         for (uint32_t c = 0; c < chunks; ++c) {
             float* slot = ws + ((size_t)(first + c) * p.heads + a) * elems + e;
@@ -295,7 +297,8 @@ uzu_status retention(hipStream_t s, const RetentionParams& p) {
         else if (per <= 64) UZU_LOC(64);
         else UZU_LOC(128);
 #undef UZU_LOC
-        UZU_PROPAGATE(launch_check([&] { hipLaunchKernelGGL(retention_chunk_scan_kernel, grid, dim3(256), 0, s, p, p.chunk_ws); }, "retention_chunk_scan"));
+        const dim3 sgrid(p.nseq, p.heads, std::min<uint32_t>((p.dim * p.vdim + 255) / 256, 1024));
+        UZU_PROPAGATE(launch_check([&] { hipLaunchKernelGGL(retention_chunk_scan_kernel, sgrid, dim3(256), 0, s, p, p.chunk_ws); }, "retention_chunk_scan"));
         return launch_check([&] { hipLaunchKernelGGL(retention_chunk_out_kernel, cgrid, dim3(256), 0, s, p, (const float*)p.chunk_ws); }, "retention_chunk_out");
     }
 #define UZU_RET(N) return launch_check([&] { hipLaunchKernelGGL(retention_steps_kernel<N>, grid, dim3(256), 0, s, p); }, "retention")

@@ -25,7 +25,9 @@ __device__ __forceinline__ void split_bf16(float a, float b, uint32_t& hi, uint3
     hi = (uint32_t)h0 | ((uint32_t)h1 << 16), lo = (uint32_t)l0 | ((uint32_t)l1 << 16);
 }
 
-template <int NB> // dim and vdim padded to RP = 32 NB
+// SPLIT (few items, many keys: decode steps): grid.z workgroups share an item tile's key blocks (block i goes to workgroup i mod grid.z) and leave unnormalised
+// sums with their running maximum / denominator in p.split_ws; window_attention_merge_kernel combines them.  The sink belongs to split 0.
+template <int NB, bool SPLIT> // dim and vdim padded to RP = 32 NB
 __global__ void __launch_bounds__(256) window_attention_mfma_kernel(WindowAttentionParams p) {
     constexpr int RP = 32 * NB, KP = RP * 2 + 16, TP = 80, VEC = RP / 8;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -74,8 +76,9 @@ __global__ void __launch_bounds__(256) window_attention_mfma_kernel(WindowAttent
             qh[s] = fh, ql[s] = fl;
         }
     }
-    float m_run = p.sinks ? p.sinks[head] : -1.0e30f;
-    float l_run = p.sinks ? 1.0f : 0.0f;
+    const bool with_sink = p.sinks && (!SPLIT || blockIdx.z == 0);
+    float m_run = with_sink ? p.sinks[head] : -1.0e30f;
+    float l_run = with_sink ? 1.0f : 0.0f;
     f32x16_t o[NB];
 #pragma unroll
     for (int b = 0; b < NB; ++b)
@@ -86,7 +89,8 @@ __global__ void __launch_bounds__(256) window_attention_mfma_kernel(WindowAttent
     const size_t kpitch = (size_t)p.kv_heads * p.dim, vpitch = (size_t)p.kv_heads * p.vdim;
     const float inv_cap = p.soft_cap != 0.0f ? 1.0f / p.soft_cap : 0.0f;
 
-    for (uint32_t kb = kmin; kb <= kmax; kb += 32) {
+    const uint32_t kstep = SPLIT ? 32 * gridDim.z : 32;
+    for (uint32_t kb = kmin + (SPLIT ? 32 * blockIdx.z : 0); kb <= kmax; kb += kstep) {
         __syncthreads(); // the block before has been read
         for (uint32_t v = tid; v < 32 * VEC; v += 256) {
             const uint32_t key = v / VEC, e0 = (v % VEC) * 8, kk = kb + key;
@@ -160,6 +164,16 @@ __global__ void __launch_bounds__(256) window_attention_mfma_kernel(WindowAttent
         }
     }
     if (!valid) return;
+    if (SPLIT) {
+        float* ws = p.split_ws + (((size_t)(sp.row0 + row) * p.heads + head) * gridDim.z + blockIdx.z) * (RP + 4);
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4)
+                *(f32x4_v*)(ws + b * 32 + 8 * g4 + 4 * half) = f32x4_v{o[b][4 * g4], o[b][4 * g4 + 1], o[b][4 * g4 + 2], o[b][4 * g4 + 3]};
+        if (half == 0) ws[RP] = m_run, ws[RP + 1] = l_run;
+        return;
+    }
     const float inv = 1.0f / l_run;
     float* out = p.out + ((size_t)(sp.row0 + row) * p.heads + head) * p.vdim;
 #pragma unroll
@@ -171,6 +185,21 @@ __global__ void __launch_bounds__(256) window_attention_mfma_kernel(WindowAttent
         }
 }
 
+// a workgroup per item: out = sum_s e^(m_s - M) O_s / sum_s e^(m_s - M) l_s over the splits, in split order (a split that saw no key has l = 0 and m = -1e30)
+__global__ void __launch_bounds__(128) window_attention_merge_kernel(const float* ws, float* out, uint32_t splits, uint32_t vdim, uint32_t rp) {
+    const uint32_t item = blockIdx.x, tid = threadIdx.x;
+    const float* base = ws + (size_t)item * splits * (rp + 4);
+    float M = -1.0e30f;
+    for (uint32_t s = 0; s < splits; ++s) M = fmaxf(M, base[(size_t)s * (rp + 4) + rp]);
+    float den = 0.0f;
+    for (uint32_t s = 0; s < splits; ++s) den = fmaf(fast_exp(base[(size_t)s * (rp + 4) + rp] - M), base[(size_t)s * (rp + 4) + rp + 1], den);
+    for (uint32_t c = tid; c < vdim; c += 128) {
+        float acc = 0.0f;
+        for (uint32_t s = 0; s < splits; ++s) acc = fmaf(fast_exp(base[(size_t)s * (rp + 4) + rp] - M), base[(size_t)s * (rp + 4) + c], acc);
+        out[(size_t)item * vdim + c] = acc / den;
+    }
+}
+
 uint32_t blocks_of(const WindowAttentionParams& p) {
     const uint32_t w = p.dim > p.vdim ? p.dim : p.vdim;
     return w <= 32 ? 1 : w <= 64 ? 2 : w <= 128 ? 4 : 0;
@@ -178,18 +207,36 @@ uint32_t blocks_of(const WindowAttentionParams& p) {
 
 } // namespace
 
-// bf16 caches, head widths that are multiples of 8 up to 128 (16-byte rows), prompt-sized passes (a decode step's few items would leave the tiles empty)
+size_t window_attention_split_ws_bytes(uint32_t rows, uint32_t heads, uint32_t splits) { return (size_t)rows * heads * splits * (128 + 4) * 4; }
+
+// bf16 caches, head widths that are multiples of 8 up to 128 (16-byte rows); prompt-sized passes, or a decode-sized pass with a workspace to split its keys
+// (without one a decode step's few items would walk all their keys in one nearly empty workgroup: the simple form does that better)
+static bool use_split(const WindowAttentionParams& p) {
+    return p.splits > 1 && p.splits <= 64 && p.split_ws && p.split_ws_bytes >= window_attention_split_ws_bytes(p.rows, p.heads, p.splits);
+}
+
 bool window_attention_mfma_supported(const WindowAttentionParams& p) {
+    const bool split = use_split(p);
     return p.cache_bf16 && blocks_of(p) && p.dim % 8 == 0 && p.vdim % 8 == 0 && p.ldq % 4 == 0 && p.kv_heads && p.heads % p.kv_heads == 0 && p.nseq && p.tiles &&
-           p.rows >= 16 * p.nseq && p.kv_heads <= 65535 && ((uintptr_t)p.q & 15) == 0 && ((uintptr_t)p.out & 15) == 0;
+           (split || p.rows >= 16 * p.nseq) && p.kv_heads <= 65535 && ((uintptr_t)p.q & 15) == 0 && ((uintptr_t)p.out & 15) == 0;
 }
 
 uzu_status window_attention_mfma(hipStream_t s, const WindowAttentionParams& p) {
     UZU_REQUIRE(window_attention_mfma_supported(p), "window_attention: the matrix-core form does not take this shape");
     const uint32_t nb = blocks_of(p);
-    const dim3 grid(p.tiles, p.kv_heads);
     const size_t lds = (size_t)32 * (32 * nb * 2 + 16) + (size_t)32 * nb * 80;
-#define UZU_WA(NB) return launch_check([&] { hipLaunchKernelGGL(window_attention_mfma_kernel<NB>, grid, dim3(256), lds, s, p); }, "window_attention_mfma")
+    if (use_split(p)) {
+        const dim3 grid(p.tiles, p.kv_heads, p.splits);
+#define UZU_WA(NB) UZU_PROPAGATE(launch_check([&] { hipLaunchKernelGGL((window_attention_mfma_kernel<NB, true>), grid, dim3(256), lds, s, p); }, "window_attention_mfma_split"))
+        if (nb == 1) UZU_WA(1);
+        else if (nb == 2) UZU_WA(2);
+        else UZU_WA(4);
+#undef UZU_WA
+        return launch_check([&] { hipLaunchKernelGGL(window_attention_merge_kernel, dim3(p.rows * p.heads), dim3(128), 0, s, (const float*)p.split_ws, p.out, p.splits, p.vdim, 32 * nb); },
+                            "window_attention_merge");
+    }
+    const dim3 grid(p.tiles, p.kv_heads);
+#define UZU_WA(NB) return launch_check([&] { hipLaunchKernelGGL((window_attention_mfma_kernel<NB, false>), grid, dim3(256), lds, s, p); }, "window_attention_mfma")
     if (nb == 1) UZU_WA(1);
     if (nb == 2) UZU_WA(2);
     UZU_WA(4);

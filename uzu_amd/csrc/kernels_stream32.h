@@ -189,7 +189,13 @@ struct WindowAttentionParams {
     uint32_t form;  // 0: chosen by shape; 1: the simple form (a wave per row and head); 2: the matrix-core form
     uint32_t nseq;  // entries of `spans`
     uint32_t tiles; // sum over the sequences of ceil(count * (heads / kv_heads) / 128): the matrix-core form's item tiles (the caller knows the counts)
+    // matrix-core form, few rows over many keys (decode): `splits` > 1 workgroups share the key blocks of an item tile, partial sums go through split_ws
+    // (window_attention_split_ws_bytes(rows, heads, splits) bytes) and a merge launch.  0 / null: one workgroup walks all keys of its tile.
+    uint32_t splits;
+    float* split_ws;
+    size_t split_ws_bytes;
 };
+size_t window_attention_split_ws_bytes(uint32_t rows, uint32_t heads, uint32_t splits);
 bool window_attention_mfma_supported(const WindowAttentionParams& p);
 uzu_status window_attention(hipStream_t s, const WindowAttentionParams& p);
 

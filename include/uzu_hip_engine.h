@@ -144,6 +144,9 @@ uzu_status uzu_hip_s32_window_attention(uzu_hip_context* ctx, const float* q, co
                                         uint32_t heads, uint32_t kv_heads, uint32_t dim, uint32_t vdim, uint32_t window, float scale, float soft_cap, uint32_t cache_bf16, uint32_t form);
 uzu_status uzu_hip_s32_retention(uzu_hip_context* ctx, const float* q, const float* k, const float* v, const float* decay, float* state_inout, float* out, uint32_t rows,
                                  uint32_t start, uint32_t heads, uint32_t dim, uint32_t vdim, uint32_t form);
+/* 1: the full library.  0: the `stream32` flavor (make -C uzu_amd/csrc stream32 -> libuzu_hip_stream32.so), built without the fused decode kernels of the
+ * bf16-stream models -- four minutes of compile time that a first use serving only an f32-stream design does not need; it refuses bf16-stream models at creation. */
+int uzu_hip_decode_kernels_present(void);
 /* LanguageModelState reset: context length 0, DeltaNet conv / SSM state zeroed. */
 uzu_status uzu_hip_model_reset(uzu_hip_model* m);
 uint32_t uzu_hip_model_context_length(const uzu_hip_model* m);

@@ -25,12 +25,30 @@ class UzuHipError(RuntimeError):
 STATUS_NAMES = {0: "OK", 1: "INVALID_ARGUMENT", 2: "UNSUPPORTED", 3: "HIP", 4: "OUT_OF_MEMORY", 5: "STATE"}
 
 
+STREAM32_LIB_PATH = os.path.join(_HERE, "lib", "libuzu_hip_stream32.so")
+
+
 def build(force: bool = False, jobs: int = 8) -> str:
     """Compile every HIP source for gfx950 (hipcc cross-compiles without a GPU)."""
     if force:
         subprocess.run(["make", "-C", CSRC, "clean"], check=True, stdout=subprocess.DEVNULL)
     subprocess.run(["make", "-C", CSRC, f"-j{jobs}"], check=True, stdout=subprocess.DEVNULL)
     return LIB_PATH
+
+
+def build_stream32(jobs: int = 8) -> str:
+    """The library without the fused decode kernels of the bf16-stream models (csrc/Makefile: stream32): what an f32-stream design needs, in a fraction of the
+    full build's time.  `use_library` makes it the library of this process."""
+    subprocess.run(["make", "-C", CSRC, f"-j{jobs}", "stream32"], check=True, stdout=subprocess.DEVNULL)
+    return STREAM32_LIB_PATH
+
+
+def use_library(path: str) -> None:
+    """Load `path` instead of LIB_PATH; before the first call into the library."""
+    global LIB_PATH, _lib
+    if _lib is not None and path != LIB_PATH:
+        raise RuntimeError("the HIP library is loaded already")
+    LIB_PATH = path
 
 
 class Buf(C.Structure):

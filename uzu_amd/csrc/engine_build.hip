@@ -303,6 +303,8 @@ void rope_tables(const uzu_rope_desc& r, uint32_t n_pos, std::vector<float>& cos
 } // namespace eng
 } // namespace uzu
 
+extern "C" int uzu_hip_decode_kernels_present(void); // k_decode.hip: 1; k_decode_absent.hip: 0
+
 extern "C" {
 
 // sizes of the description structs this library was built with (include/uzu_model_desc.h: they are part of the ABI -- uzu_layer_desc is an array element)
@@ -324,6 +326,8 @@ uzu_status uzu_hip_model_create_tp(uzu_hip_context* ctx, const uzu_model_desc* d
         UZU_UNSUPPORTED(comm != nullptr, "model_create: f32-stream designs are not sharded (single GPU only)");
         return s32_create(ctx, desc, flags, out);
     }
+    UZU_UNSUPPORTED(!uzu_hip_decode_kernels_present(), "model_create: this library is the `stream32` flavor (f32-stream designs only, built without the fused decode kernels of the "
+                                                       "bf16-stream models); run `make -C uzu_amd/csrc` for the full library");
     UZU_UNSUPPORTED(flags & UZU_MODEL_FULL_F32, "model_create: UZU_MODEL_FULL_F32 is a precision of the f32-stream designs; this model's stream is bf16");
     for (uint32_t l = 0; l < desc->num_layers; ++l)
         UZU_UNSUPPORTED(desc->layers[l].mixer_kind == UZU_MIXER_LATENT_ATTENTION || desc->layers[l].mixer_kind == UZU_MIXER_RETENTION || desc->layers[l].parallel_block ||

@@ -1888,6 +1888,8 @@ uzu_status attn_merge(hipStream_t s, const float* partials, const float* sums, c
 } // namespace k
 } // namespace uzu
 
+// 1 here; 0 in the `stream32` flavor of the library, where k_decode_absent.hip stands in for this file and bf16-stream models are refused at creation
+extern "C" int uzu_hip_decode_kernels_present(void) { return 1; }
 // tests / A-B runs: -1 = environment / default, 0 = attn_dec + attn_merge, 1 = fused (decided when a step is encoded or captured)
 extern "C" void uzu_hip_debug_set_attn_fused(int mode) { uzu::k::g_attn_fused_override = mode; }
 #ifdef UZU_ATTN_FUSED_BUILD

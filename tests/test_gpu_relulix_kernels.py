@@ -216,11 +216,12 @@ def test_score_cap_bounds_a_huge_score(hip_ctx):
             assert abs(got - want) < 1e-5, (cap, got, want)
 
 
-RET = [(2, 8, 8, 5, 0), (3, 16, 24, 70, 0), (1, 64, 64, 200, 0), (4, 24, 8, 129, 0), (2, 128, 128, 64, 0), (2, 8, 40, 33, 50), (5, 12, 20, 1, 9)]
+RET = [(2, 8, 8, 5, 0), (3, 16, 24, 70, 0), (1, 64, 64, 200, 0), (4, 24, 8, 129, 0), (2, 128, 128, 64, 0), (2, 8, 40, 33, 50), (5, 12, 20, 1, 9), (2, 96, 72, 150, 30),
+       (1, 136, 16, 70, 0), (1, 100, 128, 65, 3)]
 
 
 @pytest.mark.parametrize("H,dim,vd,T,start", RET)
-@pytest.mark.parametrize("form", [1, 2])
+@pytest.mark.parametrize("form", [1, 2, 3])
 def test_retention_both_forms_against_the_recurrence(hip_ctx, H, dim, vd, T, start, form):
     rng = np.random.default_rng(H + T)
     q, k, v = rng.standard_normal((T, H, dim)), rng.standard_normal((T, H, dim)) / np.sqrt(dim), rng.standard_normal((T, H, vd))
@@ -232,7 +233,7 @@ def test_retention_both_forms_against_the_recurrence(hip_ctx, H, dim, vd, T, sta
     assert np.abs(got - want).max() < 3e-5 * np.abs(want).max() and np.abs(gs - S).max() < 3e-5 * np.abs(S).max()
 
 
-@pytest.mark.parametrize("form", [1, 2])
+@pytest.mark.parametrize("form", [1, 2, 3])
 def test_retention_state_carries_a_far_token_through_portions(hip_ctx, form):
     """One early token writes a large outer product into a slowly decaying head; 500 positions later a query along its key reads its value back, scaled by
     decay^distance -- across portions of 64, 1, 2, 200, ... rows that hand the state on.  The fast head has forgotten it."""

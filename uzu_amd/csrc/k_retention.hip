@@ -254,6 +254,167 @@ __global__ void __launch_bounds__(256) retention_chunk_out_kernel(RetentionParam
     }
 }
 
+// ---- the chunk kernels on the matrix cores with f32 operands (v_mfma_f32_32x32x2_f32: products and sums in f32, nothing is rounded to bf16), head widths up
+// to 128.  Lane l of a wave feeds A[row l % 32][k = l / 32] and B[k = l / 32][column l % 32]; its 16 results are rows 8 (r / 4) + 4 (l / 32) + r % 4 of column l % 32.
+typedef float f32x16_m __attribute__((ext_vector_type(16)));
+
+// A_c = (decayed keys)^T values: [dim][vdim] from 64 rows; tiles of 32 x 32 dealt round-robin to the four waves (at most four each)
+__global__ void __launch_bounds__(256) retention_chunk_local_mfma_kernel(RetentionParams p, float* ws) {
+    extern __shared__ float s_kv[]; // [64][KP] decayed keys, then [64][VP] values, zero-padded
+    __shared__ float s_pw[kChunk + 1];
+    uint32_t z, c;
+    SeqSpan sp;
+    if (!find_chunk(p, blockIdx.x, z, c, sp)) return;
+    const uint32_t a = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5, dim = p.dim, vdim = p.vdim;
+    const uint32_t TI = (dim + 31) / 32, TJ = (vdim + 31) / 32, KP = 32 * TI, VP = 32 * TJ;
+    const uint32_t r0 = sp.row0 + c * kChunk, n = sp.count - c * kChunk < kChunk ? sp.count - c * kChunk : kChunk;
+    if (tid == 0) {
+        float w = 1.0f;
+        const float decay = p.decay[a];
+        for (uint32_t t = 0; t <= kChunk; ++t) s_pw[t] = w, w *= decay;
+    }
+    __syncthreads();
+    float* s_k = s_kv;
+    float* s_v = s_kv + (size_t)kChunk * KP;
+    for (uint32_t e = tid; e < kChunk * KP; e += 256) {
+        const uint32_t t = e / KP, i = e % KP;
+        s_k[e] = (t < n && i < dim) ? p.qkv[(size_t)(r0 + t) * p.ld + p.k_col + a * dim + i] * s_pw[n - 1 - t] : 0.0f;
+    }
+    for (uint32_t e = tid; e < kChunk * VP; e += 256) {
+        const uint32_t t = e / VP, j = e % VP;
+        s_v[e] = (t < n && j < vdim) ? p.qkv[(size_t)(r0 + t) * p.ld + p.v_col + a * vdim + j] : 0.0f;
+    }
+    __syncthreads();
+    f32x16_m acc[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[q][r] = 0.0f;
+    const uint32_t tiles = TI * TJ, steps = (n + 1) / 2;
+    for (uint32_t t2 = 0; t2 < steps; ++t2) {
+        const uint32_t t = 2 * t2 + half;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const uint32_t tt = wave + 4 * q;
+            if (tt < tiles) acc[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(s_k[t * KP + (tt / TJ) * 32 + l32], s_v[t * VP + (tt % TJ) * 32 + l32], acc[q], 0, 0, 0);
+        }
+    }
+    float* dst = ws + ((size_t)blockIdx.x * p.heads + a) * dim * vdim;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const uint32_t tt = wave + 4 * q;
+        if (tt >= tiles) continue;
+        const uint32_t j = (tt % TJ) * 32 + l32;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const uint32_t i = (tt / TJ) * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+            if (i < dim && j < vdim) dst[(size_t)i * vdim + j] = acc[q][r];
+        }
+    }
+}
+
+// o_i = decay^(i+1) S_c^T q_i + sum_(j <= i) decay^(i-j) <q_i, k_j> v_j for the 64 rows of a chunk
+__global__ void __launch_bounds__(256) retention_chunk_out_mfma_kernel(RetentionParams p, const float* ws) {
+    constexpr uint32_t SW = 64, SP = SW + 1;        // a slab of 64 key coordinates, pitch 65: rows on distinct banks
+    __shared__ float s_buf[2 * kChunk * SP];        // query slab + key slab; later the values [64][VP <= 128]
+    __shared__ float s_p[kChunk][kChunk + 1], s_pw[kChunk + 2];
+    uint32_t z, c;
+    SeqSpan sp;
+    if (!find_chunk(p, blockIdx.x, z, c, sp)) return;
+    const uint32_t a = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5, dim = p.dim, vdim = p.vdim;
+    const uint32_t TJ = (vdim + 31) / 32, VP = 32 * TJ;
+    const uint32_t r0 = sp.row0 + c * kChunk, n = sp.count - c * kChunk < kChunk ? sp.count - c * kChunk : kChunk;
+    if (tid == 0) {
+        float w = 1.0f;
+        const float decay = p.decay[a];
+        for (uint32_t t = 0; t <= kChunk + 1; ++t) s_pw[t] = w, w *= decay;
+    }
+    const float* qb = p.qkv + (size_t)r0 * p.ld + p.q_col + a * dim;
+    const float* kb = p.qkv + (size_t)r0 * p.ld + p.k_col + a * dim;
+    const float* vb = p.qkv + (size_t)r0 * p.ld + p.v_col + a * vdim;
+    float* s_q = s_buf;
+    float* s_k = s_buf + kChunk * SP;
+    // scores of the chunk's rows among themselves: wave w owns the 32 x 32 tile (w / 2, w % 2)
+    const uint32_t pi = wave >> 1, pj = wave & 1;
+    f32x16_m sc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sc[r] = 0.0f;
+    for (uint32_t d0 = 0; d0 < dim; d0 += SW) {
+        __syncthreads();
+        for (uint32_t e = tid; e < kChunk * SW; e += 256) {
+            const uint32_t r = e / SW, dd = e % SW, d = d0 + dd;
+            const bool ok = r < n && d < dim;
+            s_q[r * SP + dd] = ok ? qb[(size_t)r * p.ld + d] : 0.0f;
+            s_k[r * SP + dd] = ok ? kb[(size_t)r * p.ld + d] : 0.0f;
+        }
+        __syncthreads();
+        const uint32_t dn = dim - d0 < SW ? dim - d0 : SW;
+        for (uint32_t d = 0; d < dn; d += 2) sc = __builtin_amdgcn_mfma_f32_32x32x2f32(s_q[(pi * 32 + l32) * SP + d + half], s_k[(pj * 32 + l32) * SP + d + half], sc, 0, 0, 0);
+    }
+    __syncthreads(); // the slabs are done with, s_pw is there
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const uint32_t i = pi * 32 + 8 * (r >> 2) + 4 * half + (r & 3), j = pj * 32 + l32;
+        s_p[i][j] = (j <= i && i < n) ? sc[r] * s_pw[i - j] : 0.0f;
+    }
+    float* s_v = s_buf; // [64][VP]
+    for (uint32_t e = tid; e < kChunk * VP; e += 256) {
+        const uint32_t t = e / VP, j = e % VP;
+        s_v[e] = (t < n && j < vdim) ? vb[(size_t)t * p.ld + j] : 0.0f;
+    }
+    __syncthreads();
+    // outputs: tiles (row half oi, column tile oc), dealt round-robin to the waves (at most two each)
+    const uint32_t tiles = 2 * TJ;
+    f32x16_m o[2];
+#pragma unroll
+    for (int q = 0; q < 2; ++q)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[q][r] = 0.0f;
+    const uint32_t steps = (n + 1) / 2;
+    for (uint32_t j2 = 0; j2 < steps; ++j2) {
+        const uint32_t j = 2 * j2 + half;
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            const uint32_t tt = wave + 4 * q;
+            if (tt < tiles) o[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(s_p[(tt / TJ) * 32 + l32][j], s_v[j * VP + (tt % TJ) * 32 + l32], o[q], 0, 0, 0);
+        }
+    }
+    if (sp.start || c) { // the carried state: + sum_d (decay^(i+1) q_i[d]) S[d][column], the state's rows straight from memory
+        const float* S = ws + ((size_t)blockIdx.x * p.heads + a) * dim * vdim;
+        for (uint32_t d0 = 0; d0 < dim; d0 += SW) {
+            __syncthreads(); // the values (first slab) / the slab before have been read
+            for (uint32_t e = tid; e < kChunk * SW; e += 256) {
+                const uint32_t r = e / SW, dd = e % SW, d = d0 + dd;
+                s_q[r * SP + dd] = (r < n && d < dim) ? qb[(size_t)r * p.ld + d] * s_pw[r + 1] : 0.0f;
+            }
+            __syncthreads();
+            const uint32_t dn = dim - d0 < SW ? dim - d0 : SW;
+            for (uint32_t d = 0; d < dn; d += 2) {
+                const uint32_t dg = d0 + d + half;
+#pragma unroll
+                for (int q = 0; q < 2; ++q) {
+                    const uint32_t tt = wave + 4 * q;
+                    if (tt >= tiles) continue;
+                    const uint32_t col = (tt % TJ) * 32 + l32;
+                    const float sv = (dg < dim && col < vdim) ? S[(size_t)dg * vdim + col] : 0.0f;
+                    o[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(s_q[((tt / TJ) * 32 + l32) * SP + d + half], sv, o[q], 0, 0, 0);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+        const uint32_t tt = wave + 4 * q;
+        if (tt >= tiles) continue;
+        const uint32_t col = (tt % TJ) * 32 + l32;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const uint32_t i = (tt / TJ) * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+            if (i < n && col < vdim) p.out[((size_t)(r0 + i) * p.heads + a) * vdim + col] = o[q][r];
+        }
+    }
+}
+
 // a wave per (row, head)
 __global__ void __launch_bounds__(64) head_rms_gate_kernel(float* x, const float* gate, uint32_t ldg, float eps, uint32_t heads, uint32_t width) {
     const uint32_t r = blockIdx.x, a = blockIdx.y, lane = threadIdx.x;
@@ -284,8 +445,16 @@ uzu_status retention(hipStream_t s, const RetentionParams& p) {
     UZU_REQUIRE(p.heads <= 65535, "retention: too many heads for one launch");
     const uint32_t parts = 256 / p.vdim, per = (p.dim + parts - 1) / parts;
     const dim3 grid(p.nseq, p.heads);
-    if (p.form == 2 || (p.form == 0 && p.chunk_ws && p.rows > 16 * p.nseq)) { // prompt-sized: in chunks
+    if (p.form == 2 || p.form == 3 || (p.form == 0 && p.chunk_ws && p.rows > 16 * p.nseq)) { // prompt-sized: in chunks (3: without the matrix cores)
         UZU_REQUIRE(p.chunk_ws && p.chunks && p.chunk_ws_bytes >= retention_chunk_ws_bytes(p.chunks, p.heads, p.dim, p.vdim), "retention: the chunked form needs its workspace");
+        if (p.form != 3 && p.dim <= 128 && p.vdim <= 128) { // on the matrix cores with f32 operands
+            const dim3 cgrid(p.chunks, p.heads);
+            const size_t lds = (size_t)kChunk * (32 * ((p.dim + 31) / 32) + 32 * ((p.vdim + 31) / 32)) * 4;
+            UZU_PROPAGATE(launch_check([&] { hipLaunchKernelGGL(retention_chunk_local_mfma_kernel, cgrid, dim3(256), lds, s, p, p.chunk_ws); }, "retention_chunk_local_mfma"));
+            const dim3 sgrid(p.nseq, p.heads, std::min<uint32_t>((p.dim * p.vdim + 255) / 256, 1024));
+            UZU_PROPAGATE(launch_check([&] { hipLaunchKernelGGL(retention_chunk_scan_kernel, sgrid, dim3(256), 0, s, p, p.chunk_ws); }, "retention_chunk_scan"));
+            return launch_check([&] { hipLaunchKernelGGL(retention_chunk_out_mfma_kernel, cgrid, dim3(256), 0, s, p, (const float*)p.chunk_ws); }, "retention_chunk_out_mfma");
+        }
         uint32_t stage = 16384 / (p.dim + p.vdim);
         stage = stage >= 64 ? 64 : stage >= 32 ? 32 : stage >= 16 ? 16 : 8;
         const dim3 cgrid(p.chunks, p.heads);

@@ -203,7 +203,8 @@ uzu_status window_attention(hipStream_t s, const WindowAttentionParams& p);
 // v_col; q and k rotated and k scaled already):   S <- decay[a] S + k v^T,   out[r, a, :] = S^T q.
 // states: device array [nseq] of pointers to f32 [heads][dim][vdim], the sequences' states, read at the pass's first row (zero instead when the span starts at
 // position 0) and left behind its last.  Every sum runs in the same order whatever else the pass carries.  form 0: chosen by the sequence's row count; 1: token
-// by token; 2: in chunks of 64 rows (scores of the chunk's own rows + the carried state, a decayed state update per chunk).
+// by token; 2: in chunks of 64 rows (scores of the chunk's own rows + the carried state, a decayed state update per chunk; head widths up to 128 on the matrix
+// cores with f32 operands); 3: the chunks without the matrix cores.
 struct RetentionParams {
     const float* qkv;
     uint32_t ld, q_col, k_col, v_col;

@@ -1,7 +1,6 @@
 """Relulix through the engine (HipModel: states, batched steps, prefill / decode, sampling, the generate loops) against the float64 oracle on small models of
 the tests' own making: odd sizes, head widths that differ between keys and values, grouped and single key / value heads, layers with and without window /
 cap / scaling / experts / shared caches, retention layers in front, between and behind attention layers, one and several winners."""
-import os
 
 import numpy as np
 import pytest

@@ -26,58 +26,9 @@ from typing import Dict, List, Optional, Tuple
 import numpy as np
 
 from . import desc as D
+from .design_tensors import Tensors as _Tensors, bits_to_f32 as _bits_to_f32, f32_to_bf16_bits as _f32_to_bf16_bits, full_linear as _full
 
 ARCHITECTURE = "Lazolix"
-
-
-def _f32_to_bf16_bits(a: np.ndarray) -> np.ndarray:
-    """round-to-nearest-even bf16 bit patterns of an f32 array"""
-    u = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32).astype(np.uint64)
-    r = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
-    return r
-
-
-def _bits_to_f32(bits: np.ndarray) -> np.ndarray:
-    return (bits.astype(np.uint32) << 16).view(np.float32)
-
-
-class _Tensors:
-    """bf16 tensors of a safetensors file by name: `bits(name)` = uint16 patterns, `f32(name)` = their values; shapes are checked where the caller knows them."""
-
-    def __init__(self, st, err):
-        self.st, self.err = st, err
-
-    def has(self, name: str) -> bool:
-        return name in self.st.index
-
-    def shape(self, name: str) -> Tuple[int, ...]:
-        if name not in self.st.index:
-            raise self.err(f"{self.st.path}: tensor '{name}' not found")
-        return tuple(self.st.index[name][1])
-
-    def bits(self, name: str, shape: Optional[Tuple[int, ...]] = None) -> np.ndarray:
-        have = self.shape(name)
-        dtype = self.st.index[name][0]
-        if shape is not None and tuple(shape) != have:
-            raise self.err(f"{self.st.path}: tensor '{name}' is {list(have)}, the configuration implies {list(shape)}")
-        if dtype == "BF16":
-            return np.ascontiguousarray(self.st.tensor(name, have, "BF16"))
-        if dtype == "F32":
-            return _f32_to_bf16_bits(self.st.tensor(name, have, "F32"))
-        raise self.err(f"{self.st.path}: tensor '{name}' is {dtype}: bf16 (or f32) expected")
-
-    def f32(self, name: str, shape: Optional[Tuple[int, ...]] = None) -> np.ndarray:
-        have = self.shape(name)
-        if self.st.index[name][0] == "F32":
-            if shape is not None and tuple(shape) != have:
-                raise self.err(f"{self.st.path}: tensor '{name}' is {list(have)}, the configuration implies {list(shape)}")
-            return np.ascontiguousarray(self.st.tensor(name, have, "F32"))
-        return np.ascontiguousarray(_bits_to_f32(self.bits(name, shape)))
-
-
-def _full(bits: np.ndarray, bias: Optional[np.ndarray] = None) -> D.LinearWeights:
-    n, k = bits.shape
-    return D.LinearWeights(n=int(n), k=int(k), bits=16, group_size=0, method=D.QUANT_NONE, weights=np.ascontiguousarray(bits), out_biases=bias)
 
 
 def _dyn_tanh(t: _Tensors, name: str, width: int, eps: float) -> D.NormWeights:

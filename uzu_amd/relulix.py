@@ -27,7 +27,7 @@ from typing import Dict, List, Optional
 import numpy as np
 
 from . import desc as D
-from .lazolix import _Tensors, _bits_to_f32, _f32_to_bf16_bits, _full
+from .design_tensors import Tensors as _Tensors, bits_to_f32 as _bits_to_f32, f32_to_bf16_bits as _f32_to_bf16_bits, full_linear as _full
 
 ARCHITECTURE = "Relulix"
 GATE_ALPHA = 1.702  # the sigmoid's slope in an expert's gate
